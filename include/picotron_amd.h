@@ -1,0 +1,178 @@
+/*
+ * picotron_amd -- C ABI of the MI355X (gfx950) hot-path library  libpicotron_amd.so
+ *
+ * picotron has no FFI of its own: the path it accelerates is a set of Python functions
+ * (picotron/context_parallel/context_parallel.py, picotron/model.py) that call torch /
+ * flash-attn ops.  Each entry point below replaces the arithmetic of one of those call
+ * sites; the citation after "replaces:" is the reference file:line.
+ *
+ * Conventions
+ *  - plain pointers to DEVICE memory + sizes; no torch types.  The library never allocates,
+ *    frees or synchronises: every call only enqueues kernels on `stream` (a hipStream_t,
+ *    passed as void*; NULL = the default stream).  Safe to call from any host thread.
+ *  - every function returns PICO_OK (0) or a negative pico_status; the text of the last
+ *    failure on the calling thread is available from pico_last_error().
+ *  - tensors are addressed as [B, H, S, D] with explicit element strides for (b, h, s) and a
+ *    unit stride on D, so both a contiguous [B,H,S,D] buffer and a transposed view of a
+ *    [B,S,H,D] buffer (what picotron's Attention produces, model.py:128-130) are accepted.
+ *  - dtype codes: PICO_BF16 / PICO_F32.  Attention operands are bf16 only.
+ */
+#ifndef PICOTRON_AMD_H
+#define PICOTRON_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum pico_status {
+  PICO_OK = 0,
+  PICO_ERR_NULL = -1,      /* a required pointer is NULL */
+  PICO_ERR_DTYPE = -2,     /* unsupported dtype code */
+  PICO_ERR_SHAPE = -3,     /* unsupported size (head_dim, hidden, negative dims, GQA ratio) */
+  PICO_ERR_ALIGN = -4,     /* pointer or stride not aligned as the kernel needs */
+  PICO_ERR_STRIDE = -5,    /* stride combination not supported */
+  PICO_ERR_WORKSPACE = -6, /* workspace too small */
+  PICO_ERR_LAUNCH = -7     /* hipLaunchKernel reported an error */
+} pico_status;
+
+typedef enum pico_dtype { PICO_BF16 = 0, PICO_F32 = 1 } pico_dtype;
+
+/* Library version string, e.g. "picotron_amd 0.1 gfx950". */
+const char* pico_version(void);
+/* Message of the last failing call made by this thread ("" if none). */
+const char* pico_last_error(void);
+
+/* ------------------------------------------------------------------ RMSNorm
+ * replaces: LlamaRMSNorm.forward  model.py:81-86  (cast_then_scale = 1: the normalised value is
+ *           rounded to the io dtype, then multiplied by the weight in that dtype)
+ *           TritonRMSNorm.forward model.py:51-65 -> flash-attn layer_norm_fn(is_rms_norm=True)
+ *           (cast_then_scale = 0: fp32 maths, one rounding).
+ * x, y: [rows, hidden] contiguous, dtype `dtype`; weight: [hidden] same dtype.
+ * rstd: optional [rows] fp32 output (1/sqrt(mean x^2 + eps)), saved for the backward.
+ * residual_in / residual_out: optional fused pre-norm residual add (TritonRMSNorm's
+ *   residual= / prenorm= arguments): h = x + residual_in is normalised and, if residual_out is
+ *   given, written there in the io dtype.  Pass NULL for both to get the plain norm.
+ * hidden must be a multiple of 8 (bf16) / 4 (fp32) and <= 16384.
+ */
+int pico_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd,
+                     const void* residual_in, void* residual_out,
+                     int64_t rows, int64_t hidden, float eps, int cast_then_scale,
+                     int dtype, void* stream);
+
+/* Bytes of fp32 workspace pico_rmsnorm_bwd needs for the per-block partial sums of dweight. */
+int64_t pico_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t hidden);
+
+/* replaces: autograd of model.py:81-86 / the Triton backward of layer_norm_fn.
+ * dx = rstd * (g - xhat * mean(g * xhat)),  g = dy * w,  xhat = x * rstd;  dweight = sum_rows dy * xhat.
+ * x is the tensor that was normalised (after the residual add, if any).
+ * dx: [rows, hidden] `dtype`; dweight: [hidden] fp32; workspace: device scratch of at least
+ * pico_rmsnorm_bwd_workspace_bytes() bytes (contents undefined on entry and exit).
+ */
+int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
+                     void* dx, float* dweight, void* workspace, int64_t workspace_bytes,
+                     int64_t rows, int64_t hidden, int dtype, void* stream);
+
+/* ------------------------------------------------------------------ RoPE
+ * replaces: apply_rotary_pos_emb  model.py:12-19  and the flash-attn rotary call model.py:136-137
+ *           (non-interleaved: element i pairs with i + D/2), with the row selection of
+ *           update_rope_for_context_parallel  context_parallel.py:189-195 folded in as pos_offset.
+ * y[b,h,s,:D/2] = x1*cos - x2*sin ; y[b,h,s,D/2:] = x2*cos + x1*sin,  cos/sin row = pos_offset + s.
+ * cos, sin: [>= pos_offset + S, table_ld] tables of dtype table_dtype; only the first D/2 columns
+ * are read (get_cos_sin duplicates the halves, model.py:31).  x and y may alias (in place).
+ * inverse = 1 applies the rotation by -theta, which is the backward (adjoint) of the forward.
+ * D must be a multiple of 16 and <= 256; strides in elements, D contiguous.
+ */
+int pico_rope(const void* x, void* y, const void* cos, const void* sin,
+              int64_t B, int64_t H, int64_t S, int64_t D,
+              int64_t x_stride_b, int64_t x_stride_h, int64_t x_stride_s,
+              int64_t y_stride_b, int64_t y_stride_h, int64_t y_stride_s,
+              int64_t table_ld, int64_t pos_offset, int inverse,
+              int table_dtype, int dtype, void* stream);
+
+/* ------------------------------------------------------------------ SwiGLU activation
+ * replaces: F.silu(gate) * up  model.py:186  and its autograd.
+ * gate, up, y (and dy, dgate, dup): [rows, cols] with row pitches *_ld in elements; cols % 8 == 0.
+ */
+int pico_swiglu_fwd(const void* gate, const void* up, void* y,
+                    int64_t rows, int64_t cols, int64_t gate_ld, int64_t up_ld, int64_t y_ld,
+                    int dtype, void* stream);
+int pico_swiglu_bwd(const void* dy, const void* gate, const void* up, void* dgate, void* dup,
+                    int64_t rows, int64_t cols, int64_t dy_ld, int64_t gate_ld, int64_t up_ld,
+                    int64_t dgate_ld, int64_t dup_ld, int dtype, void* stream);
+
+/* ------------------------------------------------------------------ online-softmax merge
+ * replaces: update_out_and_lse  context_parallel.py:157-187 (the _update branch, :170-171):
+ *   out <- out - sigmoid(block_lse - lse) * (out - block_out);  lse <- lse - logsigmoid(lse - block_lse)
+ * out: [rows, D] fp32 in/out; lse: [rows] fp32 in/out; block_out: [rows, D] of block_dtype;
+ * block_lse: [rows] fp32.  rows = B*H*Sq.
+ */
+int pico_lse_merge(float* out, float* lse, const void* block_out, const float* block_lse,
+                   int64_t rows, int64_t D, int block_dtype, void* stream);
+
+/* ------------------------------------------------------------------ attention
+ * One descriptor serves forward and backward.  q, k, v, dout are bf16.
+ *   query i of the launch sits at absolute position q_offset + i, key j at position j;
+ *   with causal != 0 key j is visible iff j <= q_offset + i.
+ * q_offset = 0 and Sq == Sk is the masked diagonal block of the reference (context_parallel.py:116-119);
+ * causal = 0 is a dense off-diagonal block; q_offset = r*Sc with Sk = (r+1)*Sc runs ALL ring steps
+ * of cp rank r in one launch (the K/V chunks 0..r laid out consecutively along S).
+ * Hq % Hkv == 0: query head h reads kv head h / (Hq/Hkv), i.e. the effect of the reference's
+ * repeat_interleave (model.py:142-143) without the copy; pass Hkv == Hq for pre-expanded K/V.
+ */
+typedef struct pico_attn_desc {
+  int32_t B, Hq, Hkv, Sq, Sk, D;   /* D in {64, 128} */
+  int32_t causal;
+  int32_t q_offset;
+  float sm_scale;
+  int32_t reserved;
+  int64_t q_stride[3];             /* elements, order (b, h, s); D stride is 1 */
+  int64_t k_stride[3];
+  int64_t v_stride[3];
+  int64_t o_stride[3];             /* out, and dout in the backward */
+} pico_attn_desc;
+
+/* replaces: ring_attention_forward  context_parallel.py:112-128  (merge = 0), and
+ *           ring_attention_forward + update_out_and_lse  context_parallel.py:37-40 (merge = 1).
+ * out:  [B,Hq,Sq,D] addressed by o_stride; dtype out_dtype (PICO_BF16 or PICO_F32).
+ * lse:  [B,Hq,Sq] contiguous fp32.
+ * merge = 1: (out, lse) hold the running fp32 result of earlier blocks on entry (out_dtype must be
+ * PICO_F32) and the merged result on exit -- the online softmax simply continues from that state.
+ * Rows that see no key get out = 0 and lse = -inf.
+ */
+int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
+                  void* out, float* lse, int out_dtype, int merge, void* stream);
+
+/* replaces: D = sum(dO * O, dim=-1)  context_parallel.py:145.
+ * delta: [B,Hq,Sq] fp32.  out is addressed by o_stride like dout and has dtype out_dtype.
+ * If dq_acc is not NULL the [B,Hq,Sq,D] contiguous fp32 buffer is zeroed in the same pass.
+ */
+int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* dout, const void* out, int out_dtype,
+                             float* delta, float* dq_acc, void* stream);
+
+/* replaces: ring_attention_backward  context_parallel.py:130-155 and the fp32 accumulation of
+ *           RingAttentionFunc.backward  context_parallel.py:85-93.
+ * lse, delta: [B,Hq,Sq] fp32 (lse is the FINAL merged lse, as in the reference).
+ * dq_acc: [B,Hq,Sq,D] contiguous fp32, accumulated with atomic adds (zero it first, or keep the
+ *         running sum across ring steps).
+ * dk, dv: [B,Hkv,Sk,D] contiguous; dkv_dtype PICO_F32 with accumulate = 1 adds into the buffers
+ *         (the travelling fp32 accumulators of the ring), accumulate = 0 overwrites; PICO_BF16 overwrites.
+ *         With Hq > Hkv the group's query heads are reduced inside the kernel.
+ */
+int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
+                  const void* dout, const float* lse, const float* delta,
+                  float* dq_acc, void* dk, void* dv, int dkv_dtype, int accumulate, void* stream);
+
+/* fp32 -> bf16/fp32 conversion with layout change: src [B,H,S,D] contiguous fp32,
+ * dst addressed by dst_stride (b,h,s).  Used to hand dq_acc back in the dtype / layout of q.
+ * No counterpart in the reference (autograd does the cast, context_parallel.py:110).
+ */
+int pico_convert_f32(const float* src, void* dst, int64_t B, int64_t H, int64_t S, int64_t D,
+                     int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_stride_s,
+                     int dst_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PICOTRON_AMD_H */

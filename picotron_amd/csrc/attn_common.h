@@ -1,0 +1,75 @@
+// Pieces shared by the attention forward and backward kernels (gfx950, wave64, MFMA 32x32x16 bf16).
+//
+// MFMA 32x32x16 operand layout (verified on hardware): lane l, half h = l / 32, n = l % 32
+//   A[m][k]  : lane holds m = n, k = 8h .. 8h+7          (8 bf16)
+//   B[k][n]  : lane holds n,     k = 8h .. 8h+7          (8 bf16)
+//   C[m][n]  : lane holds column n, register i holds row 8*(i/4) + 4h + i%4   (16 fp32)
+// The sum over k does not care which physical index sits in slot k as long as A and B agree, so a
+// C tile can be fed back as the k-operand of the next MFMA straight from registers: registers
+// 8c .. 8c+7 of a lane hold rows {16c + 8jj + 4h + t : jj < 2, t < 4}, and the partner operand is
+// fetched with that same row order.
+//
+// ds_read_b64_tr_b16 (verified on hardware): within a group of 16 lanes, lane p supplies the address
+// of 4 consecutive 16-bit elements; lane p receives element p%4 of lanes {p/4, 4 + p/4, 8 + p/4, 12 + p/4}.
+// With lane p pointing at tile[row0 + p/4][col0 + 4*(p%4)] every lane p ends up with
+// tile[row0 .. row0+3][col0 + p]: a 4-deep column of a row-major tile, which is what an MFMA operand
+// needs when the contraction index is the tile's row.
+#pragma once
+#include "common.h"
+
+namespace pico {
+
+typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+
+// 4 rows x 1 column of a row-major bf16 tile in LDS, transposed into the lane (see header comment).
+// `p` must point at tile[row0 + (lane%16)/4][col0 + 4*(lane%4)].
+__device__ __forceinline__ s16x4 lds_read_tr(const __bf16* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(p));
+}
+
+// Two transposed reads -> the 8 k-slots of an MFMA operand.  Slots 0-3 come from rows
+// row0 .. row0+3, slots 4-7 from rows row0+8 .. row0+11 (the register order of a C tile).
+__device__ __forceinline__ bf16x8 lds_read_tr_pair(const __bf16* p, int ld) {
+  s16x4 lo = lds_read_tr(p);
+  s16x4 hi = lds_read_tr(p + 8 * ld);
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+__device__ __forceinline__ bf16x8 pack8(const f32x16& c, int base) {
+  bf16x8 r;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) r[e] = static_cast<__bf16>(c[base + e]);
+  return r;
+}
+
+// max / sum of a value across the two 32-lane halves of a wave (lane l with lane l^32)
+__device__ __forceinline__ float half_max(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_sum(float v) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+struct AttnParams {
+  const __bf16* q; const __bf16* k; const __bf16* v;
+  int B, Hq, Hkv, Sq, Sk;
+  int causal, q_offset;
+  float sm_scale;
+  int64_t qs[3], ks[3], vs[3], os[3];
+};
+
+int check_attn_desc(const char* fn, const pico_attn_desc* d);
+AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, const void* v);
+
+}  // namespace pico

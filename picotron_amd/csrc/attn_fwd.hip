@@ -1,0 +1,317 @@
+// Flash-style attention forward for gfx950: S^T = K Q^T and O^T = V^T P^T on MFMA 32x32x16 bf16.
+//
+// Computing the TRANSPOSED score tile puts one query in each lane (column n of the C tile) and
+// the keys in its registers, so the online-softmax max/sum are in-register reductions plus one
+// exchange between the two wave halves, the per-query rescale factor is a per-lane scalar for the
+// O^T accumulator, and the probabilities can be fed to the second MFMA as its B operand without
+// leaving registers.  K and V tiles are staged row-major in LDS once per workgroup; K is read with
+// 16-byte loads, V with transposing LDS reads (the contraction index of P V is V's row).
+#include "attn_common.h"
+
+namespace pico {
+namespace {
+
+struct FwdParams {
+  AttnParams a;
+  void* out;
+  float* lse;
+  int out_f32;
+  int merge;
+};
+
+template <int D, int QB, int NW>
+struct FwdCfg {
+  static constexpr int kThreads = 64 * NW;
+  static constexpr int BM = 32 * QB * NW;  // queries per workgroup
+  static constexpr int BN = 64;            // keys per LDS tile
+  static constexpr int LDK = D + 8;        // K tile pitch: 16-byte row reads hit distinct banks
+  static constexpr int LDV = D + 32;       // V tile pitch: 4 rows x 64 bytes of a transposed read do
+  static constexpr int kVecPerRow = D / 8;
+  static constexpr int kLoads = BN * kVecPerRow / kThreads;  // 16-byte loads per thread per tensor
+  static_assert(BN * kVecPerRow % kThreads == 0, "tile must split evenly over the threads");
+};
+
+template <int D, int QB, int NW>
+__global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(const FwdParams p) {
+  using C = FwdCfg<D, QB, NW>;
+  constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK, LDV = C::LDV;
+  __shared__ __attribute__((aligned(16))) __bf16 sK[BN * LDK];
+  __shared__ __attribute__((aligned(16))) __bf16 sV[BN * LDV];
+
+  const AttnParams& a = p.a;
+  const int n_qtiles = (a.Sq + BM - 1) / BM;
+  const int qtile = n_qtiles - 1 - static_cast<int>(blockIdx.x);  // causal: longest tiles first
+  const int hq = blockIdx.y, b = blockIdx.z;
+  const int hkv = hq / (a.Hq / a.Hkv);
+  const int q0 = qtile * BM;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int n = lane % 32, h = lane / 32;
+
+  const __bf16* qbase = a.q + b * a.qs[0] + hq * a.qs[1];
+  const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
+  const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
+
+  // ---- Q fragments (B operand of S^T): lane = query, 8 consecutive d per 16-wide k step
+  bf16x8 qf[QB][D / 16];
+  int qrow[QB];
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    qrow[qb] = q0 + (wave * QB + qb) * 32 + n;
+    const bool live = qrow[qb] < a.Sq;
+    const __bf16* src = qbase + static_cast<int64_t>(live ? qrow[qb] : 0) * a.qs[2] + 8 * h;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      u32x4 raw = {0, 0, 0, 0};
+      if (live) raw = *reinterpret_cast<const u32x4*>(src + 16 * s);
+      qf[qb][s] = __builtin_bit_cast(bf16x8, raw);
+    }
+  }
+
+  // ---- running state: m in the log2 domain (scores scaled by sm_scale*log2e), l split over the halves
+  const float c = a.sm_scale * kLog2e;
+  float m_run[QB], l_run[QB];
+  f32x16 o[QB][D / 32];
+  const int64_t lse_row0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq;
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.f;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
+    if (p.merge && qrow[qb] < a.Sq) {
+      // continue from (out, lse) of the earlier blocks: m = lse, l = 1, acc = out
+      const float prev = p.lse[lse_row0 + qrow[qb]];
+      if (prev != -INFINITY) {
+        m_run[qb] = prev * kLog2e;
+        l_run[qb] = (h == 0) ? 1.f : 0.f;
+        const float* po = static_cast<const float*>(p.out) + b * a.os[0] + hq * a.os[1] +
+                          static_cast<int64_t>(qrow[qb]) * a.os[2];
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const f32x4 v4 = *reinterpret_cast<const f32x4*>(po + 32 * db + 8 * j + 4 * h);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) o[qb][db][4 * j + t] = v4[t];
+          }
+      }
+    }
+  }
+
+  // ---- key range of this query tile
+  const int q_hi = (q0 + BM < a.Sq ? q0 + BM : a.Sq);           // one past the last live query
+  int kv_end = a.Sk;
+  if (a.causal) {
+    const int vis = a.q_offset + q_hi;                            // keys < vis can be seen by some query
+    kv_end = vis < a.Sk ? vis : a.Sk;
+    if (kv_end < 0) kv_end = 0;
+  }
+  const int ntiles = (kv_end + BN - 1) / BN;
+
+  // ---- global -> register staging of one K/V tile
+  u32x4 kreg[C::kLoads], vreg[C::kLoads];
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < C::kLoads; ++i) {
+      const int idx = tid + i * C::kThreads;
+      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+      const int key = k0 + r;
+      u32x4 zk = {0, 0, 0, 0}, zv = {0, 0, 0, 0};
+      if (key < a.Sk) {
+        zk = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + cv * 8);
+        zv = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + cv * 8);
+      }
+      kreg[i] = zk;
+      vreg[i] = zv;
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < C::kLoads; ++i) {
+      const int idx = tid + i * C::kThreads;
+      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = kreg[i];
+      *reinterpret_cast<u32x4*>(&sV[r * LDV + cv * 8]) = vreg[i];
+    }
+  };
+
+  if (ntiles > 0) load_tile(0);
+
+  for (int t = 0; t < ntiles; ++t) {
+    const int k0 = t * BN;
+    __syncthreads();  // everyone is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (t + 1 < ntiles) load_tile(k0 + BN);
+
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const int blk_q_lo = a.q_offset + q0 + (wave * QB + qb) * 32;  // position of the block's first query
+      if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
+      // ---- S^T[key][query] for 64 keys x 32 queries
+      f32x16 s_acc[BN / 32];
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sK[(32 * mb + n) * LDK + 16 * s + 8 * h]);
+          s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
+        }
+      }
+      // ---- mask (only for tiles that straddle the diagonal or the end of K)
+      const bool need_mask = (a.causal && k0 + BN - 1 > blk_q_lo) || (k0 + BN > a.Sk);
+      if (need_mask) {
+        const int qpos = a.causal ? a.q_offset + qrow[qb] : 0x7fffffff;
+#pragma unroll
+        for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = k0 + 32 * mb + 8 * (i / 4) + 4 * h + (i % 4);
+            if (key > qpos || key >= a.Sk) s_acc[mb][i] = -INFINITY;
+          }
+      }
+      // ---- online softmax
+      float mx = s_acc[0][0];
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
+      mx = half_max(mx);
+      const float m_new = fmaxf(m_run[qb], mx * c);
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = fast_exp2(m_run[qb] - m_use);
+      m_run[qb] = m_new;
+      float psum = 0.f;
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const float pv = fast_exp2(s_acc[mb][i] * c - m_use);
+          s_acc[mb][i] = pv;
+          psum += pv;
+        }
+      l_run[qb] = l_run[qb] * alpha + psum;
+      if (__any(alpha != 1.f)) {
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
+      }
+      // ---- O^T[d][query] += V^T[d][key] P^T[key][query]
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+          const bf16x8 pf = pack8(s_acc[mb], 8 * cc);
+          const int krow = 32 * mb + 16 * cc + 4 * h + (lane % 16) / 4;
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db) {
+            const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+            const bf16x8 vf = lds_read_tr_pair(&sV[krow * LDV + col], LDV);
+            o[qb][db] = mfma32(vf, pf, o[qb][db]);
+          }
+        }
+    }
+  }
+
+  // ---- epilogue
+#pragma unroll
+  for (int qb = 0; qb < QB; ++qb) {
+    const float l_tot = half_sum(l_run[qb]);
+    const bool live = qrow[qb] < a.Sq;
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (live && h == 0)
+      p.lse[lse_row0 + qrow[qb]] = l_tot > 0.f ? (m_run[qb] + fast_log2(l_tot)) * kLn2 : -INFINITY;
+    if (!live) continue;
+    const int64_t off = b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(qrow[qb]) * a.os[2];
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = 32 * db + 8 * j + 4 * h;
+        if (p.out_f32) {
+          f32x4 v4;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) v4[t] = o[qb][db][4 * j + t] * inv;
+          *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + off + d) = v4;
+        } else {
+          u32x2 v2;
+          v2[0] = pack_bf16x2(o[qb][db][4 * j] * inv, o[qb][db][4 * j + 1] * inv);
+          v2[1] = pack_bf16x2(o[qb][db][4 * j + 2] * inv, o[qb][db][4 * j + 3] * inv);
+          *reinterpret_cast<u32x2*>(static_cast<__bf16*>(p.out) + off + d) = v2;
+        }
+      }
+  }
+}
+
+template <int D, int QB, int NW>
+void launch(const FwdParams& p, hipStream_t s) {
+  using C = FwdCfg<D, QB, NW>;
+  const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
+  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW>), dim3(n_qtiles, p.a.Hq, p.a.B), dim3(C::kThreads), 0, s, p);
+}
+
+}  // namespace
+
+int check_attn_desc(const char* fn, const pico_attn_desc* d) {
+  if (!d) return fail(PICO_ERR_NULL, "%s: descriptor is NULL", fn);
+  if (d->D != 64 && d->D != 128) return fail(PICO_ERR_SHAPE, "%s: head_dim %d not supported (64 or 128)", fn, d->D);
+  if (d->B < 0 || d->Hq <= 0 || d->Hkv <= 0 || d->Sq < 0 || d->Sk < 0)
+    return fail(PICO_ERR_SHAPE, "%s: negative size (B=%d Hq=%d Hkv=%d Sq=%d Sk=%d)", fn, d->B, d->Hq, d->Hkv, d->Sq, d->Sk);
+  if (d->Hq % d->Hkv != 0) return fail(PICO_ERR_SHAPE, "%s: Hq=%d is not a multiple of Hkv=%d", fn, d->Hq, d->Hkv);
+  if (d->B > 65535 || d->Hq > 65535) return fail(PICO_ERR_SHAPE, "%s: B and Hq must be <= 65535", fn);
+  if (d->q_offset < 0) return fail(PICO_ERR_SHAPE, "%s: q_offset=%d must be >= 0", fn, d->q_offset);
+  if (!(d->sm_scale > 0.f)) return fail(PICO_ERR_SHAPE, "%s: sm_scale must be positive", fn);
+  const int64_t* all[4] = {d->q_stride, d->k_stride, d->v_stride, d->o_stride};
+  for (const int64_t* st : all)
+    for (int i = 0; i < 3; ++i)
+      if (st[i] < 0 || st[i] % 8 != 0)
+        return fail(PICO_ERR_STRIDE, "%s: strides must be non-negative multiples of 8 elements", fn);
+  return PICO_OK;
+}
+
+AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, const void* v) {
+  AttnParams a;
+  a.q = static_cast<const __bf16*>(q);
+  a.k = static_cast<const __bf16*>(k);
+  a.v = static_cast<const __bf16*>(v);
+  a.B = d->B; a.Hq = d->Hq; a.Hkv = d->Hkv; a.Sq = d->Sq; a.Sk = d->Sk;
+  a.causal = d->causal != 0;
+  a.q_offset = d->q_offset;
+  a.sm_scale = d->sm_scale;
+  for (int i = 0; i < 3; ++i) {
+    a.qs[i] = d->q_stride[i]; a.ks[i] = d->k_stride[i]; a.vs[i] = d->v_stride[i]; a.os[i] = d->o_stride[i];
+  }
+  return a;
+}
+
+}  // namespace pico
+
+using namespace pico;
+
+extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, void* out,
+                             float* lse, int out_dtype, int merge, void* stream) {
+  if (int rc = check_attn_desc("pico_attn_fwd", desc)) return rc;
+  if (out_dtype != PICO_BF16 && out_dtype != PICO_F32)
+    return fail(PICO_ERR_DTYPE, "pico_attn_fwd: out dtype code %d not supported", out_dtype);
+  if (merge && out_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "pico_attn_fwd: merge needs an fp32 running out");
+  if (desc->B == 0 || desc->Sq == 0) return PICO_OK;
+  if (!q || !out || !lse || (desc->Sk > 0 && (!k || !v)))
+    return fail(PICO_ERR_NULL, "pico_attn_fwd: q, k, v, out and lse are required");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
+    return fail(PICO_ERR_ALIGN, "pico_attn_fwd: q, k, v and out must be 16-byte aligned");
+  FwdParams p;
+  p.a = make_params(desc, q, k, v);
+  p.out = out;
+  p.lse = lse;
+  p.out_f32 = out_dtype == PICO_F32;
+  p.merge = merge != 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (desc->D == 64) launch<64, 1, 4>(p, s);
+  else launch<128, 1, 4>(p, s);
+  return check_launch("pico_attn_fwd");
+}

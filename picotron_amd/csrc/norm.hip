@@ -1,0 +1,343 @@
+// RMSNorm forward / backward for gfx950.  Bandwidth-bound: every element is moved with 16-byte
+// accesses, one row is owned by a wave (hidden <= 64*8 vectors) or by a 256-thread block, the row
+// stays in registers between the reduction and the normalisation so HBM is touched once.
+#include "common.h"
+
+namespace pico {
+namespace {
+
+constexpr int kFwdThreads = 256;
+constexpr int kBwdThreads = 512;
+constexpr int kMaxBwdBlocks = 256;   // rows of the dweight workspace
+constexpr int kReduceSlices = 16;
+
+template <int G>
+__device__ __forceinline__ float group_sum(float v, float* smem /* this group's 4 floats, G == 256 only */) {
+  v = wave_sum(v);
+  if constexpr (G == kWave) {
+    return v;
+  } else {
+    const int wave = (threadIdx.x % G) / kWave;
+    __syncthreads();
+    if (threadIdx.x % kWave == 0) smem[wave] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int i = 0; i < G / kWave; ++i) t += smem[i];
+    return t;
+  }
+}
+
+// y = w * round(x * rstd)  (cast_then_scale)  or  round(x * rstd * w)
+template <typename T, int G, int NV>
+__global__ __launch_bounds__(kFwdThreads) void rmsnorm_fwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ w, T* __restrict__ y, float* __restrict__ rstd,
+    const T* __restrict__ res_in, T* __restrict__ res_out, int64_t rows, int hidden, float eps,
+    int cast_then_scale) {
+  constexpr int V = io<T>::kVec;
+  __shared__ float smem[8];
+  const int gid = threadIdx.x / G;
+  const int t = threadIdx.x % G;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * (kFwdThreads / G) + gid;
+  const int nvec = hidden / V;
+  // G == 256: the block owns one row, so `row < rows` is block-uniform and the barriers inside
+  // group_sum are reached by every thread.  G == 64: no barrier is used.
+  if (row >= rows) return;
+  const T* xr = x + row * hidden;
+  float vals[NV][V];
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = t + j * G;
+    if (v < nvec) {
+      io<T>::load(xr + v * V, vals[j]);
+      if (res_in != nullptr) {
+        float r[V];
+        io<T>::load(res_in + row * hidden + v * V, r);
+#pragma unroll
+        for (int e = 0; e < V; ++e) vals[j][e] += r[e];
+        if (res_out != nullptr) io<T>::store(res_out + row * hidden + v * V, vals[j]);
+      }
+#pragma unroll
+      for (int e = 0; e < V; ++e) ss += vals[j][e] * vals[j][e];
+    }
+  }
+  ss = group_sum<G>(ss, smem + gid * 4);
+  const float r = rsqrtf(ss / static_cast<float>(hidden) + eps);
+  if (rstd != nullptr && t == 0) rstd[row] = r;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int v = t + j * G;
+    if (v < nvec) {
+      float wv[V], o[V];
+      io<T>::load(w + v * V, wv);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float n = vals[j][e] * r;
+        o[e] = cast_then_scale ? io<T>::round(n) * wv[e] : n * wv[e];
+      }
+      io<T>::store(y + row * hidden + v * V, o);
+    }
+  }
+}
+
+// dx and per-block partial sums of dweight.
+template <typename T, int G, int NV>
+__global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ rstd, T* __restrict__ dx, float* __restrict__ partial,
+    int64_t rows, int hidden) {
+  constexpr int V = io<T>::kVec;
+  constexpr int GPB = kBwdThreads / G;
+  extern __shared__ float dw_lds[];  // [hidden] when GPB > 1
+  __shared__ float smem[8];
+  const int gid = threadIdx.x / G;
+  const int t = threadIdx.x % G;
+  const int nvec = hidden / V;
+  const float inv_h = 1.f / static_cast<float>(hidden);
+  float dw[NV][V];
+#pragma unroll
+  for (int j = 0; j < NV; ++j)
+#pragma unroll
+    for (int e = 0; e < V; ++e) dw[j][e] = 0.f;
+  if constexpr (GPB > 1) {
+    for (int i = threadIdx.x; i < hidden; i += kBwdThreads) dw_lds[i] = 0.f;
+  }
+  // rows are dealt round-robin to groups; with G == 256 (GPB == 2) a group's trip count can differ
+  // from its neighbour's, so that variant pads the loop to a block-uniform count for the barriers.
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * GPB;
+  const int64_t first = static_cast<int64_t>(blockIdx.x) * GPB + gid;
+  const int64_t trips = (rows - static_cast<int64_t>(blockIdx.x) * GPB + stride - 1) / stride;  // block-uniform upper bound
+  for (int64_t it = 0; it < trips; ++it) {
+    const int64_t row = first + it * stride;
+    const bool live = row < rows;
+    float xh[NV][V], g[NV][V];
+    float c = 0.f;
+    const float r = live ? rstd[row] : 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * G;
+      if (live && v < nvec) {
+        float dyv[V], wv[V];
+        io<T>::load(x + row * hidden + v * V, xh[j]);
+        io<T>::load(dy + row * hidden + v * V, dyv);
+        io<T>::load(w + v * V, wv);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          xh[j][e] *= r;
+          g[j][e] = dyv[e] * wv[e];
+          c += g[j][e] * xh[j][e];
+          dw[j][e] += dyv[e] * xh[j][e];
+        }
+      }
+    }
+    c = group_sum<G>(c, smem + gid * 4) * inv_h;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * G;
+      if (live && v < nvec) {
+        float o[V];
+#pragma unroll
+        for (int e = 0; e < V; ++e) o[e] = r * (g[j][e] - xh[j][e] * c);
+        io<T>::store(dx + row * hidden + v * V, o);
+      }
+    }
+  }
+  float* out = partial + static_cast<int64_t>(blockIdx.x) * hidden;
+  if constexpr (GPB > 1) {
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * G;
+      if (v < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) atomicAdd(&dw_lds[v * V + e], dw[j][e]);
+      }
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < hidden; i += kBwdThreads) out[i] = dw_lds[i];
+  } else {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * G;
+      if (v < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) out[v * V + e] = dw[j][e];
+      }
+    }
+  }
+}
+
+// dweight[c] = sum_p partial[p][c]; 64 columns x 16 slices per block.
+__global__ __launch_bounds__(64 * kReduceSlices) void rmsnorm_dw_reduce_kernel(
+    const float* __restrict__ partial, float* __restrict__ dweight, int nparts, int hidden) {
+  __shared__ float red[kReduceSlices][64];
+  const int col = blockIdx.x * 64 + threadIdx.x % 64;
+  const int slice = threadIdx.x / 64;
+  float s = 0.f;
+  if (col < hidden) {
+    for (int p = slice; p < nparts; p += kReduceSlices) s += partial[static_cast<int64_t>(p) * hidden + col];
+  }
+  red[slice][threadIdx.x % 64] = s;
+  __syncthreads();
+  if (slice == 0 && col < hidden) {
+    float tot = 0.f;
+#pragma unroll
+    for (int i = 0; i < kReduceSlices; ++i) tot += red[i][threadIdx.x];
+    dweight[col] = tot;
+  }
+}
+
+int bwd_blocks(int64_t rows, int gpb) {
+  int64_t need = (rows + gpb - 1) / gpb;
+  if (need < 1) need = 1;
+  return static_cast<int>(need < kMaxBwdBlocks ? need : kMaxBwdBlocks);
+}
+
+// smallest supported NV >= need, or 0
+int pick_nv(int need, int max_nv) {
+  for (int nv = 1; nv <= max_nv; nv *= 2)
+    if (nv >= need) return nv;
+  return 0;
+}
+
+template <typename T, int G, int NV>
+void launch_fwd(const void* x, const void* w, void* y, float* rstd, const void* ri, void* ro, int64_t rows,
+                int hidden, float eps, int cts, hipStream_t s) {
+  const int gpb = kFwdThreads / G;
+  const unsigned grid = static_cast<unsigned>((rows + gpb - 1) / gpb);
+  hipLaunchKernelGGL((rmsnorm_fwd_kernel<T, G, NV>), dim3(grid), dim3(kFwdThreads), 0, s,
+                     static_cast<const T*>(x), static_cast<const T*>(w), static_cast<T*>(y), rstd,
+                     static_cast<const T*>(ri), static_cast<T*>(ro), rows, hidden, eps, cts);
+}
+
+template <typename T, int G, int NV>
+void launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, float* partial,
+                int blocks, int64_t rows, int hidden, hipStream_t s) {
+  const size_t lds = (kBwdThreads / G > 1) ? static_cast<size_t>(hidden) * sizeof(float) : 0;
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, G, NV>), dim3(blocks), dim3(kBwdThreads), lds, s,
+                     static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), rstd,
+                     static_cast<T*>(dx), partial, rows, hidden);
+}
+
+template <typename T>
+int dispatch_fwd(const void* x, const void* w, void* y, float* rstd, const void* ri, void* ro, int64_t rows,
+                 int hidden, float eps, int cts, hipStream_t s) {
+  const int nvec = hidden / io<T>::kVec;
+  const int nv_wave = pick_nv((nvec + 63) / 64, 8);
+#define PICO_FWD(G, NV) launch_fwd<T, G, NV>(x, w, y, rstd, ri, ro, rows, hidden, eps, cts, s); return PICO_OK
+  if (nv_wave) {
+    switch (nv_wave) {
+      case 1: PICO_FWD(64, 1);
+      case 2: PICO_FWD(64, 2);
+      case 4: PICO_FWD(64, 4);
+      default: PICO_FWD(64, 8);
+    }
+  }
+  switch (pick_nv((nvec + 255) / 256, 16)) {
+    case 4: PICO_FWD(256, 4);
+    case 8: PICO_FWD(256, 8);
+    case 16: PICO_FWD(256, 16);
+    default: break;
+  }
+#undef PICO_FWD
+  return fail(PICO_ERR_SHAPE, "pico_rmsnorm_fwd: hidden=%d too large", hidden);
+}
+
+template <typename T>
+int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, float* partial,
+                 int64_t rows, int hidden, hipStream_t s, int* blocks_out) {
+  const int nvec = hidden / io<T>::kVec;
+  const int nv_wave = pick_nv((nvec + 63) / 64, 8);
+#define PICO_BWD(G, NV)                                                            \
+  {                                                                                \
+    const int blocks = bwd_blocks(rows, kBwdThreads / G);                          \
+    *blocks_out = blocks;                                                          \
+    launch_bwd<T, G, NV>(dy, x, w, rstd, dx, partial, blocks, rows, hidden, s);    \
+    return PICO_OK;                                                                \
+  }
+  if (nv_wave) {
+    switch (nv_wave) {
+      case 1: PICO_BWD(64, 1);
+      case 2: PICO_BWD(64, 2);
+      case 4: PICO_BWD(64, 4);
+      default: PICO_BWD(64, 8);
+    }
+  }
+  switch (pick_nv((nvec + 255) / 256, 8)) {
+    case 4: PICO_BWD(256, 4);
+    case 8: PICO_BWD(256, 8);
+    default: break;
+  }
+#undef PICO_BWD
+  return fail(PICO_ERR_SHAPE, "pico_rmsnorm_bwd: hidden=%d too large", hidden);
+}
+
+int check_common(const char* fn, int64_t rows, int64_t hidden, int dtype) {
+  if (dtype != PICO_BF16 && dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: dtype code %d not supported", fn, dtype);
+  const int vec = dtype == PICO_BF16 ? 8 : 4;
+  if (rows < 0 || hidden <= 0 || hidden > 16384 || hidden % vec != 0)
+    return fail(PICO_ERR_SHAPE, "%s: rows=%lld hidden=%lld (hidden must be a positive multiple of %d, <= 16384)", fn,
+                static_cast<long long>(rows), static_cast<long long>(hidden), vec);
+  return PICO_OK;
+}
+
+}  // namespace
+}  // namespace pico
+
+using namespace pico;
+
+extern "C" int pico_rmsnorm_fwd(const void* x, const void* weight, void* y, float* rstd, const void* residual_in,
+                                void* residual_out, int64_t rows, int64_t hidden, float eps, int cast_then_scale,
+                                int dtype, void* stream) {
+  if (int rc = check_common("pico_rmsnorm_fwd", rows, hidden, dtype)) return rc;
+  if (rows == 0) return PICO_OK;
+  if (!x || !weight || !y) return fail(PICO_ERR_NULL, "pico_rmsnorm_fwd: x, weight and y are required");
+  if (residual_out && !residual_in) return fail(PICO_ERR_NULL, "pico_rmsnorm_fwd: residual_out without residual_in");
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(y) || !aligned16(residual_in) || !aligned16(residual_out))
+    return fail(PICO_ERR_ALIGN, "pico_rmsnorm_fwd: pointers must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int rc = dtype == PICO_BF16
+               ? dispatch_fwd<__bf16>(x, weight, y, rstd, residual_in, residual_out, rows, static_cast<int>(hidden), eps, cast_then_scale, s)
+               : dispatch_fwd<float>(x, weight, y, rstd, residual_in, residual_out, rows, static_cast<int>(hidden), eps, cast_then_scale, s);
+  if (rc) return rc;
+  return check_launch("pico_rmsnorm_fwd");
+}
+
+extern "C" int64_t pico_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t hidden) {
+  (void)rows;
+  if (hidden <= 0) return 0;
+  return static_cast<int64_t>(kMaxBwdBlocks) * hidden * static_cast<int64_t>(sizeof(float));
+}
+
+extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd, void* dx,
+                                float* dweight, void* workspace, int64_t workspace_bytes, int64_t rows,
+                                int64_t hidden, int dtype, void* stream) {
+  if (int rc = check_common("pico_rmsnorm_bwd", rows, hidden, dtype)) return rc;
+  if (!dweight) return fail(PICO_ERR_NULL, "pico_rmsnorm_bwd: dweight is required");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (rows == 0) {  // empty sum: dweight = 0 (the reduce kernel with no partials writes zeros)
+    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + 63) / 64)),
+                       dim3(64 * kReduceSlices), 0, s, static_cast<const float*>(nullptr), dweight, 0,
+                       static_cast<int>(hidden));
+    return check_launch("pico_rmsnorm_bwd(empty)");
+  }
+  if (!dy || !x || !weight || !rstd || !dx || !workspace)
+    return fail(PICO_ERR_NULL, "pico_rmsnorm_bwd: dy, x, weight, rstd, dx and workspace are required");
+  if (workspace_bytes < pico_rmsnorm_bwd_workspace_bytes(rows, hidden))
+    return fail(PICO_ERR_WORKSPACE, "pico_rmsnorm_bwd: workspace has %lld bytes, needs %lld",
+                static_cast<long long>(workspace_bytes),
+                static_cast<long long>(pico_rmsnorm_bwd_workspace_bytes(rows, hidden)));
+  if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(workspace))
+    return fail(PICO_ERR_ALIGN, "pico_rmsnorm_bwd: pointers must be 16-byte aligned");
+  int blocks = 0;
+  float* partial = static_cast<float*>(workspace);
+  int rc = dtype == PICO_BF16
+               ? dispatch_bwd<__bf16>(dy, x, weight, rstd, dx, partial, rows, static_cast<int>(hidden), s, &blocks)
+               : dispatch_bwd<float>(dy, x, weight, rstd, dx, partial, rows, static_cast<int>(hidden), s, &blocks);
+  if (rc) return rc;
+  if (int lrc = check_launch("pico_rmsnorm_bwd")) return lrc;
+  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + 63) / 64)),
+                     dim3(64 * kReduceSlices), 0, s, partial, dweight, blocks, static_cast<int>(hidden));
+  return check_launch("pico_rmsnorm_bwd(dweight reduce)");
+}

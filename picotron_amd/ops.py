@@ -1,0 +1,275 @@
+"""Tensor-level wrappers over the C ABI: they validate, allocate outputs with torch and pass raw
+device pointers + the current HIP stream.  No arithmetic happens here and nothing falls back to
+torch ops: a CPU tensor or a missing library is an error.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import PICO_BF16, PICO_F32, AttnDesc, check
+
+_DT = {torch.bfloat16: PICO_BF16, torch.float32: PICO_F32}
+
+
+def _dt(t: torch.Tensor, what: str) -> int:
+    if t.dtype not in _DT:
+        raise RuntimeError(f"{what}: dtype {t.dtype} not supported by the HIP kernels (bf16 / fp32 only)")
+    return _DT[t.dtype]
+
+
+def _dev(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("picotron_amd kernels run on the GPU only: got a CPU tensor (there is no CPU fallback)")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+# ------------------------------------------------------------------------------- RMSNorm
+def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float, cast_then_scale: bool,
+                residual: Optional[torch.Tensor] = None, want_residual_out: bool = False,
+                want_rstd: bool = True):
+    """Returns (y, rstd or None, residual_out or None); x is [..., hidden]."""
+    _dev(x, weight, residual)
+    hidden = x.size(-1)
+    xc = x.contiguous()
+    w = weight.to(x.dtype).contiguous() if weight.dtype != x.dtype else weight.contiguous()
+    rows = xc.numel() // hidden if hidden else 0
+    y = torch.empty_like(xc)
+    rstd = torch.empty(rows, dtype=torch.float32, device=x.device) if want_rstd else None
+    res = residual.contiguous() if residual is not None else None
+    if res is not None and (res.dtype != x.dtype or res.shape != x.shape):
+        raise RuntimeError("rmsnorm_fwd: residual must match x in dtype and shape")
+    res_out = torch.empty_like(xc) if (res is not None and want_residual_out) else None
+    check(_lib.lib().pico_rmsnorm_fwd(_ptr(xc), _ptr(w), _ptr(y), _ptr(rstd), _ptr(res), _ptr(res_out), rows, hidden,
+                                      float(eps), int(cast_then_scale), _dt(x, "rmsnorm_fwd"), _stream()))
+    return y, rstd, res_out
+
+
+def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
+    """Returns (dx in x.dtype, dweight fp32 [hidden])."""
+    _dev(dy, x, weight, rstd)
+    hidden = x.size(-1)
+    xc, dyc = x.contiguous(), dy.contiguous()
+    if dyc.dtype != xc.dtype:
+        dyc = dyc.to(xc.dtype)
+    w = weight.to(x.dtype).contiguous() if weight.dtype != x.dtype else weight.contiguous()
+    rows = xc.numel() // hidden if hidden else 0
+    dx = torch.empty_like(xc)
+    dw = torch.empty(hidden, dtype=torch.float32, device=x.device)
+    ws_bytes = _lib.lib().pico_rmsnorm_bwd_workspace_bytes(rows, hidden)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
+    check(_lib.lib().pico_rmsnorm_bwd(_ptr(dyc), _ptr(xc), _ptr(w), _ptr(rstd), _ptr(dx), _ptr(dw), _ptr(ws), ws_bytes,
+                                      rows, hidden, _dt(x, "rmsnorm_bwd"), _stream()))
+    return dx, dw
+
+
+# ------------------------------------------------------------------------------- RoPE
+def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos_offset: int = 0, inverse: bool = False,
+         out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rotates x [B,H,S,D] (any b/h/s strides, unit D stride) with table rows pos_offset + s."""
+    _dev(x, cos, sin, out)
+    if x.dim() != 4:
+        raise RuntimeError("rope: x must be [B, H, S, D]")
+    if x.stride(-1) != 1:
+        x = x.contiguous()
+    if cos.dtype != sin.dtype or cos.stride(-1) != 1 or sin.stride(-1) != 1 or cos.stride(0) != sin.stride(0):
+        raise RuntimeError("rope: cos and sin must share dtype and row pitch, with contiguous rows")
+    B, H, S, D = x.shape
+    if cos.size(0) < pos_offset + S:
+        raise RuntimeError(f"rope: tables have {cos.size(0)} rows, need {pos_offset + S}")
+    if out is None:
+        # keep the memory order of x so that a transposed view stays a free view downstream
+        out = torch.empty_strided(x.shape, x.stride(), dtype=x.dtype, device=x.device) if _dense(x) else torch.empty_like(x)
+    check(_lib.lib().pico_rope(_ptr(x), _ptr(out), _ptr(cos), _ptr(sin), B, H, S, D,
+                               x.stride(0), x.stride(1), x.stride(2), out.stride(0), out.stride(1), out.stride(2),
+                               cos.stride(0), int(pos_offset), int(inverse), _dt(cos, "rope tables"), _dt(x, "rope"),
+                               _stream()))
+    return out
+
+
+def _dense(t: torch.Tensor) -> bool:
+    """True if t's strides are a permutation of a contiguous layout (no gaps, no overlap)."""
+    dims = sorted(range(t.dim()), key=lambda i: t.stride(i), reverse=True)
+    expect = 1
+    for i in reversed(dims):
+        if t.size(i) != 1 and t.stride(i) != expect:
+            return False
+        expect *= t.size(i)
+    return True
+
+
+# ------------------------------------------------------------------------------- SwiGLU
+def _as_2d(t: torch.Tensor) -> torch.Tensor:
+    if t.stride(-1) != 1:
+        t = t.contiguous()
+    if t.dim() == 2:
+        return t
+    try:
+        return t.view(-1, t.size(-1))
+    except RuntimeError:
+        return t.contiguous().view(-1, t.size(-1))
+
+
+def swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    _dev(gate, up)
+    if gate.shape != up.shape or gate.dtype != up.dtype:
+        raise RuntimeError("swiglu_fwd: gate and up must match")
+    g2, u2 = _as_2d(gate), _as_2d(up)
+    y = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    y2 = y.view(-1, y.size(-1))
+    check(_lib.lib().pico_swiglu_fwd(_ptr(g2), _ptr(u2), _ptr(y2), g2.size(0), g2.size(1), g2.stride(0), u2.stride(0),
+                                     y2.stride(0), _dt(gate, "swiglu_fwd"), _stream()))
+    return y
+
+
+def swiglu_bwd(dy: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
+    _dev(dy, gate, up)
+    g2, u2, d2 = _as_2d(gate), _as_2d(up), _as_2d(dy.to(gate.dtype))
+    dg = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    du = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    dg2, du2 = dg.view(-1, dg.size(-1)), du.view(-1, du.size(-1))
+    check(_lib.lib().pico_swiglu_bwd(_ptr(d2), _ptr(g2), _ptr(u2), _ptr(dg2), _ptr(du2), g2.size(0), g2.size(1),
+                                     d2.stride(0), g2.stride(0), u2.stride(0), dg2.stride(0), du2.stride(0),
+                                     _dt(gate, "swiglu_bwd"), _stream()))
+    return dg, du
+
+
+# ------------------------------------------------------------------------------- lse merge
+def lse_merge_(out: torch.Tensor, lse: torch.Tensor, block_out: torch.Tensor, block_lse: torch.Tensor) -> None:
+    """In place: (out fp32 [..., D], lse fp32 [...]) <- merge with (block_out, block_lse)."""
+    _dev(out, lse, block_out, block_lse)
+    if out.dtype != torch.float32 or lse.dtype != torch.float32 or block_lse.dtype != torch.float32:
+        raise RuntimeError("lse_merge_: out, lse and block_lse must be fp32")
+    if not (out.is_contiguous() and lse.is_contiguous()):
+        raise RuntimeError("lse_merge_: out and lse must be contiguous (they are updated in place)")
+    D = out.size(-1)
+    rows = out.numel() // D
+    bo, bl = block_out.contiguous(), block_lse.contiguous()
+    check(_lib.lib().pico_lse_merge(_ptr(out), _ptr(lse), _ptr(bo), _ptr(bl), rows, D, _dt(bo, "lse_merge_"), _stream()))
+
+
+# ------------------------------------------------------------------------------- attention
+def _desc(q, k, v, o, sm_scale, causal, q_offset) -> AttnDesc:
+    B, Hq, Sq, D = q.shape
+    Hkv, Sk = k.size(1), k.size(2)
+    d = AttnDesc()
+    d.B, d.Hq, d.Hkv, d.Sq, d.Sk, d.D = B, Hq, Hkv, Sq, Sk, D
+    d.causal, d.q_offset, d.sm_scale = int(bool(causal)), int(q_offset), float(sm_scale)
+    for name, t in (("q_stride", q), ("k_stride", k), ("v_stride", v), ("o_stride", o)):
+        arr = getattr(d, name)
+        arr[0], arr[1], arr[2] = t.stride(0), t.stride(1), t.stride(2)
+    return d
+
+
+def _attn_in(t: torch.Tensor, what: str) -> torch.Tensor:
+    if t.dtype != torch.bfloat16:
+        raise RuntimeError(f"attention: {what} must be bf16 (got {t.dtype}); the MFMA kernels are bf16 only")
+    if t.dim() != 4:
+        raise RuntimeError(f"attention: {what} must be [B, H, S, D]")
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:3]):
+        t = t.contiguous()
+    return t
+
+
+def empty_bshd(B: int, H: int, S: int, D: int, dtype, device) -> torch.Tensor:
+    """A [B,H,S,D]-shaped view of a fresh [B,S,H,D] buffer: `.transpose(1,2).reshape(B,S,H*D)` on it is free."""
+    return torch.empty(B, S, H, D, dtype=dtype, device=device).transpose(1, 2)
+
+
+def attn_fwd(q, k, v, sm_scale: float, causal: bool, q_offset: int = 0, out: Optional[torch.Tensor] = None,
+             lse: Optional[torch.Tensor] = None, merge: bool = False, out_dtype=torch.bfloat16,
+             bshd_out: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """softmax(q k^T * scale + mask) v for q [B,Hq,Sq,D], k/v [B,Hkv,Sk,D]; returns (out, lse fp32 [B,Hq,Sq]).
+
+    merge=True continues the online softmax from the running fp32 (out, lse) passed in and updates them in place.
+    """
+    _dev(q, k, v, out, lse)
+    q, k, v = _attn_in(q, "q"), _attn_in(k, "k"), _attn_in(v, "v")
+    B, Hq, Sq, D = q.shape
+    if k.shape != v.shape or k.size(0) != B or k.size(3) != D:
+        raise RuntimeError(f"attention: shape mismatch q{tuple(q.shape)} k{tuple(k.shape)} v{tuple(v.shape)}")
+    if merge:
+        if out is None or lse is None or out.dtype != torch.float32:
+            raise RuntimeError("attn_fwd(merge=True) needs the running fp32 out and lse")
+    if out is None:
+        out = empty_bshd(B, Hq, Sq, D, out_dtype, q.device) if bshd_out else torch.empty(B, Hq, Sq, D, dtype=out_dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+    if not lse.is_contiguous() or lse.dtype != torch.float32 or out.stride(-1) != 1:
+        raise RuntimeError("attn_fwd: lse must be contiguous fp32 and out must have a unit D stride")
+    d = _desc(q, k, v, out, sm_scale, causal, q_offset)
+    check(_lib.lib().pico_attn_fwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _dt(out, "attn_fwd out"),
+                                   int(merge), _stream()))
+    return out, lse
+
+
+def attn_bwd_preprocess(dout: torch.Tensor, out: torch.Tensor, dq_acc: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """delta = sum(dout * out, -1) as fp32 [B,H,S]; zeroes dq_acc (fp32 contiguous [B,H,S,D]) if given."""
+    _dev(dout, out, dq_acc)
+    dout = _attn_in(dout, "dout")
+    if out.stride() != dout.stride():
+        out = _like_strided(out, dout)
+    B, H, S, D = dout.shape
+    delta = torch.empty(B, H, S, dtype=torch.float32, device=dout.device)
+    d = _desc(dout, dout, dout, dout, 1.0, False, 0)
+    if dq_acc is not None and not (dq_acc.is_contiguous() and dq_acc.dtype == torch.float32):
+        raise RuntimeError("attn_bwd_preprocess: dq_acc must be contiguous fp32")
+    check(_lib.lib().pico_attn_bwd_preprocess(ctypes.byref(d), _ptr(dout), _ptr(out), _dt(out, "attn out"), _ptr(delta),
+                                              _ptr(dq_acc), _stream()))
+    return delta
+
+
+def _like_strided(t: torch.Tensor, ref: torch.Tensor) -> torch.Tensor:
+    """Copy of t laid out with ref's strides (so one stride triple describes both)."""
+    r = torch.empty_strided(ref.shape, ref.stride(), dtype=t.dtype, device=t.device)
+    r.copy_(t)
+    return r
+
+
+def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset: int, dq_acc: torch.Tensor,
+             dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None, accumulate: bool = False,
+             dkv_dtype=torch.float32):
+    """Adds this block's dq into dq_acc (fp32, atomics) and writes / accumulates dk, dv [B,Hkv,Sk,D]."""
+    _dev(dout, q, k, v, lse, delta, dq_acc, dk, dv)
+    q, k, v, dout = _attn_in(q, "q"), _attn_in(k, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
+    B, Hkv, Sk, D = k.shape
+    if dk is None:
+        dk = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
+        dv = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
+        if accumulate:
+            raise RuntimeError("attn_bwd: accumulate=True needs existing dk / dv")
+    if not (dk.is_contiguous() and dv.is_contiguous() and dq_acc.is_contiguous()) or dk.dtype != dv.dtype:
+        raise RuntimeError("attn_bwd: dq_acc, dk and dv must be contiguous")
+    if dq_acc.dtype != torch.float32 or lse.dtype != torch.float32 or delta.dtype != torch.float32:
+        raise RuntimeError("attn_bwd: dq_acc, lse and delta must be fp32")
+    d = _desc(q, k, v, dout, sm_scale, causal, q_offset)
+    check(_lib.lib().pico_attn_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(lse.contiguous()),
+                                   _ptr(delta.contiguous()), _ptr(dq_acc), _ptr(dk), _ptr(dv), _dt(dk, "dk/dv"),
+                                   int(accumulate), _stream()))
+    return dk, dv
+
+
+def convert_f32(src: torch.Tensor, dtype, like: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp32 contiguous [B,H,S,D] -> dtype, laid out like `like` (same strides) or contiguous."""
+    _dev(src, like)
+    if src.dtype != torch.float32 or not src.is_contiguous() or src.dim() != 4:
+        raise RuntimeError("convert_f32: src must be a contiguous fp32 [B,H,S,D] tensor")
+    B, H, S, D = src.shape
+    if like is not None and _dense(like) and like.stride(-1) == 1:
+        dst = torch.empty_strided(src.shape, like.stride(), dtype=dtype, device=src.device)
+    else:
+        dst = torch.empty(src.shape, dtype=dtype, device=src.device)
+    check(_lib.lib().pico_convert_f32(_ptr(src), _ptr(dst), B, H, S, D, dst.stride(0), dst.stride(1), dst.stride(2),
+                                      _DT[dtype], _stream()))
+    return dst

@@ -1,0 +1,326 @@
+"""GPU parity: every C-ABI kernel against the CPU oracle on the same seeded inputs.
+
+Tolerances (from the acceptance criteria of the path): bf16 forward outputs max-abs <= 2e-2,
+lse <= 1e-3, gradients relative L2 <= 1e-2, all against an fp32 oracle; fp32 kernels much tighter.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import layers as OL
+from oracle import ring as OR
+
+pytestmark = pytest.mark.gpu
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g, dtype=torch.float32) * scale).to(dtype)
+
+
+def rel_l2(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def maxabs(a, b):
+    return (a.double().cpu() - b.double().cpu()).abs().max().item()
+
+
+@pytest.fixture(scope="module")
+def ops(device):
+    from picotron_amd import ops as _ops
+    return _ops
+
+
+# ------------------------------------------------------------------------------------ RMSNorm
+@pytest.mark.parametrize("rows,hidden", [(7, 576), (64, 2048), (33, 4096), (5, 8192), (3, 64), (0, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("cts", [True, False])
+def test_rmsnorm_fwd(ops, device, rows, hidden, dtype, cts):
+    x = rnd(rows, hidden, seed=1, dtype=dtype)
+    w = (1 + 0.1 * rnd(hidden, seed=2)).to(dtype)
+    y, rstd, _ = ops.rmsnorm_fwd(x.to(device), w.to(device), 1e-5, cts)
+    want = OL.rmsnorm(x, w, 1e-5, cast_then_scale=cts)
+    assert y.dtype == dtype and y.shape == x.shape
+    if rows == 0:
+        return
+    if dtype == torch.float32:
+        assert maxabs(y, want) <= 2e-5
+    else:
+        # same bf16 roundings as the oracle except where the fp32 reduction order flips a rounding
+        assert maxabs(y, want) <= 2e-2
+        assert (y.cpu() != want).float().mean().item() < 0.02
+    want_rstd = torch.rsqrt(x.float().pow(2).mean(-1) + 1e-5)
+    assert torch.allclose(rstd.cpu(), want_rstd, rtol=1e-5, atol=1e-6)
+
+
+def test_rmsnorm_fwd_residual(ops, device):
+    x, r = rnd(9, 1024, seed=3, dtype=torch.bfloat16), rnd(9, 1024, seed=4, dtype=torch.bfloat16)
+    w = (1 + 0.1 * rnd(1024, seed=5)).to(torch.bfloat16)
+    y, _, res = ops.rmsnorm_fwd(x.to(device), w.to(device), 1e-5, False, residual=r.to(device), want_residual_out=True)
+    h = x.float() + r.float()
+    assert maxabs(res, h.to(torch.bfloat16)) == 0.0
+    assert maxabs(y, OL.rmsnorm(h, w.float(), 1e-5, cast_then_scale=False)) <= 2e-2
+
+
+@pytest.mark.parametrize("rows,hidden", [(7, 576), (300, 2048), (1030, 1024), (33, 4096), (5, 8192), (0, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_bwd(ops, device, rows, hidden, dtype):
+    x, dy = rnd(rows, hidden, seed=6, dtype=dtype), rnd(rows, hidden, seed=7, dtype=dtype)
+    w = (1 + 0.1 * rnd(hidden, seed=8)).to(dtype)
+    rstd = torch.rsqrt(x.float().pow(2).mean(-1) + 1e-5)
+    dx, dw = ops.rmsnorm_bwd(dy.to(device), x.to(device), w.to(device), rstd.to(device))
+    want_dx, want_dw = OL.rmsnorm_backward(dy, x, w, 1e-5)
+    assert dw.dtype == torch.float32 and dw.shape == (hidden,)
+    if rows == 0:
+        assert dw.abs().max().item() == 0.0
+        return
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    assert rel_l2(dx, want_dx) <= tol
+    assert rel_l2(dw, want_dw) <= 1e-5
+
+
+# ------------------------------------------------------------------------------------ RoPE
+@pytest.mark.parametrize("B,H,S,D", [(2, 3, 17, 64), (1, 4, 33, 128), (1, 2, 5, 16)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("layout", ["bhsd", "bshd"])
+@pytest.mark.parametrize("table_dtype", [torch.bfloat16, torch.float32])
+def test_rope_fwd_bwd(ops, device, B, H, S, D, dtype, layout, table_dtype):
+    off = 11
+    cos, sin = OL.get_cos_sin(off + S, D, 10000.0, dtype=table_dtype)
+    if layout == "bhsd":
+        x = rnd(B, H, S, D, seed=9, dtype=dtype)
+    else:
+        x = rnd(B, S, H, D, seed=9, dtype=dtype).transpose(1, 2)
+    xd = x.to(device)
+    if layout == "bshd":
+        xd = x.transpose(1, 2).contiguous().to(device).transpose(1, 2)
+    y = ops.rope(xd, cos.to(device), sin.to(device), pos_offset=off)
+    want = OL.apply_rotary_pos_emb(x.float(), cos[off:].float(), sin[off:].float())
+    assert y.shape == x.shape and y.stride() == xd.stride()
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert maxabs(y, want) <= tol
+    back = ops.rope(xd, cos.to(device), sin.to(device), pos_offset=off, inverse=True)
+    assert maxabs(back, OL.apply_rotary_pos_emb_backward(x.float(), cos[off:].float(), sin[off:].float())) <= tol
+
+
+def test_rope_positions_are_exact(ops, device):
+    """pos_offset selects table rows exactly: rotating with offset r*Sc equals slicing the tables first."""
+    S, D, W = 32, 64, 4
+    cos, sin = OL.get_cos_sin(S, D, 10000.0)
+    x = rnd(1, 2, S // W, D, seed=10, dtype=torch.bfloat16).to(device)
+    for r in range(W):
+        c_r, s_r = OR.rope_slice(cos, sin, r, W)
+        a = ops.rope(x, cos.to(device), sin.to(device), pos_offset=r * (S // W))
+        b = ops.rope(x, c_r.contiguous().to(device), s_r.contiguous().to(device), pos_offset=0)
+        assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------ SwiGLU
+@pytest.mark.parametrize("shape", [(3, 5, 1536), (64, 8192), (1, 8), (0, 64)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_swiglu(ops, device, shape, dtype):
+    g, u, dy = (rnd(*shape, seed=s, dtype=dtype) for s in (11, 12, 13))
+    y = ops.swiglu_fwd(g.to(device), u.to(device))
+    dg, du = ops.swiglu_bwd(dy.to(device), g.to(device), u.to(device))
+    if g.numel() == 0:
+        assert y.shape == g.shape
+        return
+    want = OL.swiglu(g.float(), u.float())
+    wdg, wdu = OL.swiglu_backward(dy.float(), g.float(), u.float())
+    if dtype == torch.float32:
+        assert maxabs(y, want) <= 1e-5 and rel_l2(dg, wdg) <= 1e-5 and rel_l2(du, wdu) <= 1e-5
+    else:
+        assert rel_l2(y, want) <= 5e-3 and rel_l2(dg, wdg) <= 5e-3 and rel_l2(du, wdu) <= 5e-3
+
+
+def test_swiglu_strided_halves(ops, device):
+    """gate and up as the two halves of one [T, 2I] GEMM output (row pitch 2I)."""
+    gu = rnd(10, 256, seed=14, dtype=torch.bfloat16).to(device)
+    y = ops.swiglu_fwd(gu[:, :128], gu[:, 128:])
+    want = OL.swiglu(gu[:, :128].float().cpu(), gu[:, 128:].float().cpu())
+    assert rel_l2(y, want) <= 5e-3
+
+
+# ------------------------------------------------------------------------------------ lse merge
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("bdtype", [torch.bfloat16, torch.float32])
+def test_lse_merge(ops, device, D, bdtype):
+    rows = (2, 3, 37)
+    out, bo = rnd(*rows, D, seed=15), rnd(*rows, D, seed=16).to(bdtype)
+    lse, bl = rnd(*rows, seed=17) * 3, rnd(*rows, seed=18) * 3
+    bl[0, 0, :5] = float("-inf")           # a block that saw nothing leaves the row untouched
+    lse[1, 1, :3] = float("-inf")          # a running state that saw nothing adopts the block
+    o_d, l_d = out.to(device).clone(), lse.to(device).clone()
+    ops.lse_merge_(o_d, l_d, bo.to(device), bl.to(device))
+    w_o, w_l = OR.merge(out.clone(), lse.unsqueeze(-1).clone(), bo.float(), bl)
+    w_l = w_l.squeeze(-1)
+    assert torch.equal(o_d.cpu()[0, 0, :5], out[0, 0, :5]) and torch.equal(l_d.cpu()[0, 0, :5], lse[0, 0, :5])
+    assert maxabs(o_d.cpu()[1, 1, :3], bo.float()[1, 1, :3]) <= 1e-6
+    fin = torch.isfinite(w_l)
+    assert maxabs(l_d.cpu()[fin], w_l[fin]) <= 1e-5
+    ok = torch.isfinite(w_o).all(-1)
+    assert maxabs(o_d.cpu()[ok], w_o[ok]) <= 1e-5
+
+
+# ------------------------------------------------------------------------------------ attention forward
+def attn_inputs(B, Hq, Hkv, Sq, Sk, D, seed):
+    q = rnd(B, Hq, Sq, D, seed=seed, scale=1.0).to(torch.bfloat16)
+    k = rnd(B, Hkv, Sk, D, seed=seed + 1).to(torch.bfloat16)
+    v = rnd(B, Hkv, Sk, D, seed=seed + 2).to(torch.bfloat16)
+    return q, k, v
+
+
+def expand_kv(t, Hq):
+    return t.repeat_interleave(Hq // t.size(1), dim=1)
+
+
+FWD_CASES = [
+    # B, Hq, Hkv, Sq, Sk, D, causal, q_offset
+    (1, 2, 2, 128, 128, 64, True, 0),
+    (2, 4, 4, 256, 256, 64, True, 0),
+    (1, 2, 2, 256, 256, 64, False, 0),
+    (1, 2, 2, 128, 512, 64, True, 384),     # all ring steps of rank 3 of 4 in one launch
+    (1, 4, 2, 192, 192, 64, True, 0),       # GQA
+    (1, 2, 2, 100, 100, 64, True, 0),       # ragged
+    (1, 2, 1, 77, 203, 64, False, 0),       # ragged, rectangular, GQA
+    (1, 2, 2, 256, 256, 128, True, 0),
+    (1, 8, 2, 128, 384, 128, True, 256),
+    (1, 1, 1, 61, 130, 128, False, 0),
+    (1, 1, 1, 1, 1, 64, True, 0),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,q_offset", FWD_CASES)
+def test_attn_fwd(ops, device, B, Hq, Hkv, Sq, Sk, D, causal, q_offset):
+    q, k, v = attn_inputs(B, Hq, Hkv, Sq, Sk, D, seed=20)
+    scale = 1 / math.sqrt(D)
+    out, lse = ops.attn_fwd(q.to(device), k.to(device), v.to(device), scale, causal, q_offset)
+    want_o, want_lse = OR.full_attention_closed_form(q.float(), expand_kv(k, Hq).float(), expand_kv(v, Hq).float(),
+                                                     scale, causal, q_offset)
+    assert out.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    assert maxabs(out, want_o) <= 2e-2
+    assert maxabs(lse, want_lse) <= 1e-3
+
+
+def test_attn_fwd_block_equals_oracle_block(ops, device):
+    """The per-block entry (q_offset 0, Sq == Sk) is ring_attention_forward: diag masked, off-diag dense."""
+    q, k, v = attn_inputs(2, 3, 3, 160, 160, 64, seed=30)
+    for causal in (True, False):
+        out, lse = ops.attn_fwd(q.to(device), k.to(device), v.to(device), 0.125, causal)
+        w_o, w_l = OR.block_forward(q.float(), k.float(), v.float(), 0.125, causal)
+        assert maxabs(out, w_o) <= 2e-2 and maxabs(lse, w_l) <= 1e-3
+
+
+def test_attn_fwd_strided_q_and_bshd_out(ops, device):
+    """q as a transposed view of a [B,S,H,D] buffer (what Attention produces); out written BSHD."""
+    B, H, S, D = 2, 4, 128, 64
+    q_bshd = rnd(B, S, H, D, seed=31).to(torch.bfloat16)
+    _, k, v = attn_inputs(B, H, H, S, S, D, seed=32)
+    qd = q_bshd.to(device).transpose(1, 2)
+    assert not qd.is_contiguous()
+    out, lse = ops.attn_fwd(qd, k.to(device), v.to(device), 0.125, True, bshd_out=True)
+    assert out.transpose(1, 2).is_contiguous()
+    w_o, w_l = OR.block_forward(q_bshd.transpose(1, 2).float(), k.float(), v.float(), 0.125, True)
+    assert maxabs(out, w_o) <= 2e-2 and maxabs(lse, w_l) <= 1e-3
+
+
+@pytest.mark.parametrize("D", [64, 128])
+def test_attn_fwd_fused_merge_equals_ring(ops, device, D):
+    """Rank r's ring via per-chunk launches with the fused merge == the oracle's rank_forward."""
+    W, Sc, B, H = 4, 96, 1, 2
+    q, k, v = attn_inputs(B, H, H, W * Sc, W * Sc, D, seed=40)
+    scale = 1 / math.sqrt(D)
+    ks, vs = k.chunk(W, 2), v.chunk(W, 2)
+    for r in (0, 2, 3):
+        q_r = q[:, :, r * Sc:(r + 1) * Sc].contiguous()
+        out = torch.zeros(B, H, Sc, D, dtype=torch.float32, device=device)
+        lse = torch.full((B, H, Sc), float("-inf"), dtype=torch.float32, device=device)
+        for _, held, run, blk_causal in OR.schedule(W, r, True):
+            if run:
+                ops.attn_fwd(q_r.to(device), ks[held].contiguous().to(device), vs[held].contiguous().to(device), scale,
+                             blk_causal, 0, out=out, lse=lse, merge=True)
+        w_o, w_l = OR.rank_forward(q_r.float(), [t.float() for t in ks], [t.float() for t in vs], r, scale, True)
+        assert maxabs(out, w_o) <= 2e-2 and maxabs(lse, w_l) <= 1e-3
+
+
+# ------------------------------------------------------------------------------------ attention backward
+BWD_CASES = [
+    (1, 2, 2, 128, 128, 64, True, 0),
+    (2, 2, 2, 256, 256, 64, True, 0),
+    (1, 2, 2, 128, 256, 64, False, 0),
+    (1, 2, 2, 128, 512, 64, True, 384),
+    (1, 4, 2, 192, 192, 64, True, 0),
+    (1, 2, 1, 77, 203, 64, False, 0),
+    (1, 2, 2, 100, 100, 64, True, 0),
+    (1, 2, 2, 256, 256, 128, True, 0),
+    (1, 4, 2, 128, 384, 128, True, 256),
+    (1, 1, 1, 61, 130, 128, False, 0),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,q_offset", BWD_CASES)
+def test_attn_bwd(ops, device, B, Hq, Hkv, Sq, Sk, D, causal, q_offset):
+    q, k, v = attn_inputs(B, Hq, Hkv, Sq, Sk, D, seed=50)
+    do = rnd(B, Hq, Sq, D, seed=53).to(torch.bfloat16)
+    scale = 1 / math.sqrt(D)
+    qd, kd, vd, dod = (t.to(device) for t in (q, k, v, do))
+    out, lse = ops.attn_fwd(qd, kd, vd, scale, causal, q_offset)
+    dq_acc = torch.empty(B, Hq, Sq, D, dtype=torch.float32, device=device)
+    delta = ops.attn_bwd_preprocess(dod, out, dq_acc)
+    dk, dv = ops.attn_bwd(dod, qd, kd, vd, lse, delta, scale, causal, q_offset, dq_acc)
+    # oracle: autograd through the fp32 closed form on the same bf16-rounded inputs
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    w_o, _ = OR.full_attention_closed_form(qf, expand_kv(kf, Hq), expand_kv(vf, Hq), scale, causal, q_offset)
+    gq, gk, gv = torch.autograd.grad(w_o, (qf, kf, vf), do.float())
+    assert maxabs(delta, (do.float() * w_o.detach()).sum(-1)) <= 5e-2
+    assert rel_l2(dq_acc, gq) <= 1e-2
+    assert rel_l2(dk, gk) <= 1e-2
+    assert rel_l2(dv, gv) <= 1e-2
+
+
+def test_attn_bwd_block_with_final_lse_and_accumulate(ops, device):
+    """Ring backward of one rank: per-block launches that use the FINAL merged (out, lse), fp32 accumulation
+    of dq across blocks and of dk/dv into existing buffers -- against the oracle's rank_backward."""
+    W, Sc, B, H, D, r = 4, 64, 1, 2, 64, 2
+    q, k, v = attn_inputs(B, H, H, W * Sc, W * Sc, D, seed=60)
+    do = rnd(B, H, Sc, D, seed=63).to(torch.bfloat16)
+    ks, vs = [t.contiguous() for t in k.chunk(W, 2)], [t.contiguous() for t in v.chunk(W, 2)]
+    q_r = q[:, :, r * Sc:(r + 1) * Sc].contiguous()
+    w_o, w_l = OR.rank_forward(q_r.float(), [t.float() for t in ks], [t.float() for t in vs], r, 0.125, True)
+    w_dq, contrib = OR.rank_backward(do.float(), q_r.float(), [t.float() for t in ks], [t.float() for t in vs],
+                                     w_o, w_l, r, 0.125, True)
+    out_d, lse_d = w_o.to(torch.bfloat16).to(device), w_l.to(device)
+    dq_acc = torch.empty(B, H, Sc, D, dtype=torch.float32, device=device)
+    delta = ops.attn_bwd_preprocess(do.to(device), out_d, dq_acc)
+    for _, held, run, blk_causal in OR.schedule(W, r, True):
+        if not run:
+            continue
+        dk = torch.ones(B, H, Sc, D, dtype=torch.float32, device=device)   # pre-existing travelling accumulators
+        dv = torch.full((B, H, Sc, D), 2.0, dtype=torch.float32, device=device)
+        ops.attn_bwd(do.to(device), q_r.to(device), ks[held].to(device), vs[held].to(device), lse_d, delta, 0.125,
+                     blk_causal, 0, dq_acc, dk, dv, accumulate=True)
+        assert rel_l2(dk - 1.0, contrib[held][0]) <= 1e-2
+        assert rel_l2(dv - 2.0, contrib[held][1]) <= 1e-2
+    assert rel_l2(dq_acc, w_dq) <= 1e-2
+
+
+def test_convert_f32(ops, device):
+    src = rnd(2, 3, 5, 64, seed=70).to(device)
+    like = torch.empty(2, 5, 3, 64, dtype=torch.bfloat16, device=device).transpose(1, 2)
+    dst = ops.convert_f32(src, torch.bfloat16, like=like)
+    assert dst.stride() == like.stride() and torch.equal(dst, src.to(torch.bfloat16))
+    assert torch.equal(ops.convert_f32(src, torch.float32), src)
+
+
+def test_cpu_tensor_is_rejected(ops):
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.swiglu_fwd(torch.zeros(2, 8), torch.zeros(2, 8))
+
+
+def test_bad_head_dim_reports_error(ops, device):
+    q = torch.zeros(1, 1, 8, 32, dtype=torch.bfloat16, device=device)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        ops.attn_fwd(q, q, q, 1.0, True)
