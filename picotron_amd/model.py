@@ -1,0 +1,280 @@
+"""The Llama of ``picotron/model.py`` with its hot ops on hand-written gfx950 kernels.
+
+Class and function names, constructor arguments, forward signatures, parameter names, init
+distributions and init order are the reference's (``model.py:12-298``); what changes is what runs
+underneath:
+
+=====================================  =====================================================
+reference (file:line)                  here
+=====================================  =====================================================
+apply_rotary_pos_emb      :12-19       RoPE kernel (``pico_rope``), strided [B,H,S,D] views
+flash_attn rotary         :136-137     same kernel
+flash_attention           :33-37       MFMA attention kernels (``pico_attn_fwd`` / ``_bwd``)
+F.scaled_dot_product_attention :157    same kernels (there is no CPU / torch attention path)
+TritonRMSNorm             :39-65       RMSNorm kernel, fp32 maths + one rounding, optional
+                                       fused residual add / prenorm
+LlamaRMSNorm              :67-86       RMSNorm kernel, cast-then-scale rounding order
+F.silu(gate) * up         :186         SwiGLU kernel
+repeat_interleave (GQA)   :142-143     not materialised: the kernels index the kv head
+=====================================  =====================================================
+
+The projections, embedding and vocabulary projection stay on torch / hipBLASLt.
+Environment switches are read at call time like the reference does: ``FLASH_ATTEN`` picks the
+RMSNorm class (:218, :274) and the RoPE call shape (:127-140), ``CONTEXT_PARALLEL`` routes
+attention through the ring (:148).
+"""
+from __future__ import annotations
+
+import math
+import os
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+import picotron_amd.process_group_manager as pgm
+from picotron_amd.context_parallel import context_parallel
+from picotron_amd.functional import FlashAttnFunc, RMSNormFunc, RMSNormResidualFunc, RotaryFunc, SwiGLUFunc
+
+
+def apply_rotary_pos_emb(x, cos, sin):
+    """x [B,H,S,D] (any strides with unit D stride), cos/sin [S,D] with duplicated halves."""
+    return RotaryFunc.apply(x, cos, sin, 0)
+
+
+def get_cos_sin(seq_length, head_dim, base=500000.0):
+    """[S, D] cos / sin tables, halves duplicated; theta on the CPU, angles in fp32 on the device,
+    table dtype from ``DTYPE`` (bf16 unless set otherwise) -- the recipe of ``model.py:21-31``."""
+    assert head_dim % 2 == 0
+    exponents = torch.arange(0, head_dim, 2, dtype=torch.int64).float().to("cpu") / head_dim
+    theta = 1.0 / (base ** exponents)
+    dtype = torch.bfloat16 if os.getenv("DTYPE", "bfloat16") == "bfloat16" else torch.float32
+    local_rank = int(os.environ.get("LOCAL_RANK", "0"))
+    device = torch.device("cuda", local_rank) if os.getenv("DEVICE", "cuda") == "cuda" else torch.device("cpu")
+    position = torch.arange(seq_length).to(device).unsqueeze(1).float()
+    angle = position * theta.to(device).float()
+    return torch.cos(angle).to(dtype).repeat(1, 2), torch.sin(angle).to(dtype).repeat(1, 2)
+
+
+def flash_attention(q, k, v, causal=True):
+    """q [B,Hq,S,D], k/v [B,Hkv,S,D] -> [B,S,Hq,D] (the layout flash_attn_func returns, ``model.py:33-37``)."""
+    sm_scale = 1.0 / math.sqrt(q.size(-1))
+    return FlashAttnFunc.apply(q, k, v, sm_scale, causal).transpose(1, 2)
+
+
+class TritonRMSNorm(nn.Module):
+    """RMSNorm with fp32 maths and a single rounding; keeps the reference's class name and call shape."""
+
+    def __init__(self, hidden_size, eps=1e-5, device=None, dtype=None):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.empty(hidden_size, device=device, dtype=dtype))
+        self.register_parameter("bias", None)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        nn.init.ones_(self.weight)
+
+    def forward(self, hidden_states, residual=None, dropout_p=0.0, prenorm=False, residual_in_fp32=False,
+                return_dropout_mask=False):
+        if dropout_p != 0.0 or return_dropout_mask or residual_in_fp32:
+            raise NotImplementedError("TritonRMSNorm: dropout and fp32 residuals are not used by picotron and not built")
+        if residual is None:
+            y = RMSNormFunc.apply(hidden_states, self.weight, self.eps, False)
+            return (y, hidden_states) if prenorm else y
+        y, h = RMSNormResidualFunc.apply(hidden_states, residual, self.weight, self.eps)
+        return (y, h) if prenorm else y
+
+
+class LlamaRMSNorm(nn.Module):
+    """RMSNorm that rounds the normalised value to the input dtype before scaling (``model.py:81-86``)."""
+
+    def __init__(self, hidden_size, eps=1e-5):
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(hidden_size))
+        self.variance_epsilon = eps
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        nn.init.ones_(self.weight)
+
+    def forward(self, hidden_states):
+        return RMSNormFunc.apply(hidden_states, self.weight, self.variance_epsilon, True)
+
+
+def _fan_in_uniform_(tensor):
+    bound = math.sqrt(1 / tensor.size(1))
+    torch.nn.init.uniform_(tensor, -bound, bound)
+
+
+class Attention(nn.Module):
+    def __init__(self, config, layer_idx):
+        super().__init__()
+        mgr = pgm.process_group_manager
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_key_values = config.num_key_value_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        assert config.num_attention_heads % mgr.tp_world_size == 0, "num_attention_heads should be divisible by tp world size"
+        assert config.num_key_value_heads % mgr.tp_world_size == 0, "num_key_value_heads should be divisible by  tp world size"
+        self.num_local_heads = config.num_attention_heads // mgr.tp_world_size
+        self.num_local_kv_heads = config.num_key_value_heads // mgr.tp_world_size
+
+        self.q_proj = nn.Linear(config.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(config.hidden_size, self.num_key_values * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(config.hidden_size, self.num_key_values * self.head_dim, bias=False)
+        self.out_proj = nn.Linear(config.hidden_size, config.hidden_size, bias=False)
+        self.layer_idx = layer_idx
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        for proj in (self.q_proj, self.k_proj, self.v_proj, self.out_proj):
+            _fan_in_uniform_(proj.weight)
+
+    def forward(self, x, cos, sin, attention_mask=None, position_ids=None):
+        batch_size, seq_length, _ = x.size()
+        # [B,S,H*D] -> [B,H,S,D] views over [B,S,H,D] memory; the kernels take the strides as they are
+        q = self.q_proj(x).view(batch_size, seq_length, self.num_local_heads, self.head_dim).transpose(1, 2)
+        k = self.k_proj(x).view(batch_size, seq_length, self.num_local_kv_heads, self.head_dim).transpose(1, 2)
+        v = self.v_proj(x).view(batch_size, seq_length, self.num_local_kv_heads, self.head_dim).transpose(1, 2)
+        q = apply_rotary_pos_emb(q, cos, sin)
+        k = apply_rotary_pos_emb(k, cos, sin)
+        # GQA: no repeat_interleave -- query head h reads kv head h // (Hq/Hkv) inside the kernels
+
+        causal = True if q.size(2) == k.size(2) else False
+
+        if os.getenv("CONTEXT_PARALLEL", "0") == "1":
+            sm_scale = 1.0 / (q.size(-1) ** 0.5)
+            out = context_parallel.ring_attention(q, k, v, sm_scale, causal).transpose(1, 2)
+        else:
+            out = flash_attention(q, k, v, causal=causal)  # [B,S,H,D]
+
+        out = out.reshape(batch_size, seq_length, self.num_local_heads * self.head_dim)
+        return self.out_proj(out)
+
+
+class MLP(nn.Module):
+    def __init__(self, config) -> None:
+        super().__init__()
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        for proj in (self.up_proj, self.gate_proj, self.down_proj):
+            _fan_in_uniform_(proj.weight)
+
+    def forward(self, x):
+        return self.down_proj(SwiGLUFunc.apply(self.gate_proj(x), self.up_proj(x)))
+
+
+class FinalProjection(nn.Module):
+    def __init__(self, hidden_size, vocab_size, bias=False):
+        super().__init__()
+        self.in_features = hidden_size
+        self.out_features = vocab_size
+        self.weight = nn.Parameter(torch.empty(self.out_features, self.in_features))
+        self.bias = nn.Parameter(torch.empty(self.out_features)) if bias else None
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        bound = math.sqrt(1 / self.weight.size(1))
+        torch.nn.init.uniform_(self.weight, -bound, bound)
+        if self.bias is not None:
+            bound_b = math.sqrt(1 / self.bias.size(0)) if self.bias.dim() == 1 else bound
+            torch.nn.init.uniform_(self.bias, -bound_b, bound_b)
+
+    def forward(self, x):
+        return F.linear(x, self.weight, self.bias)
+
+
+class DecoderLayer(nn.Module):
+    """RMSNorm -> Attention -> residual -> RMSNorm -> MLP -> residual."""
+
+    def __init__(self, config, layer_idx):
+        super().__init__()
+        RMSNorm = LlamaRMSNorm if os.getenv("FLASH_ATTEN", "1") != "1" else TritonRMSNorm
+        self.input_layernorm = RMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.attention = Attention(config, layer_idx=layer_idx)
+        self.mlp = MLP(config)
+        self.layer_idx = layer_idx
+        head_dim = config.hidden_size // config.num_attention_heads
+        self.cos, self.sin = get_cos_sin(config.max_position_embeddings, head_dim=head_dim, base=config.rope_theta)
+        # context parallelism splits the sequence: keep the rows of this rank's positions
+        self.cos, self.sin = context_parallel.update_rope_for_context_parallel(self.cos, self.sin)
+
+    def forward(self, x, attention_mask=None, position_ids=None):
+        cos, sin = self.cos, self.sin
+        x = x + self.attention(self.input_layernorm(x), cos, sin, attention_mask, position_ids)
+        x = x + self.mlp(self.post_attention_layernorm(x))
+        return x
+
+
+class Embedding(nn.Module):
+    def __init__(self, num_embeddings, embedding_dim, padding_idx=None):
+        super().__init__()
+        self.num_embeddings = num_embeddings
+        self.embedding_dim = embedding_dim
+        self.padding_idx = padding_idx
+        self.weight = nn.Parameter(torch.empty(num_embeddings, embedding_dim))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        torch.nn.init.normal_(self.weight, mean=0.0, std=1.0)
+
+    def forward(self, x):
+        return F.embedding(x, self.weight, self.padding_idx)
+
+
+class Llama(nn.Module):
+    def __init__(self, config) -> None:
+        super().__init__()
+        assert config.hidden_size % config.num_attention_heads == 0
+        assert config.num_attention_heads % config.num_key_value_heads == 0
+        self.vocab_size = config.vocab_size
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_attention_heads
+        self.num_key_values = config.num_key_value_heads
+        self.head_dim = self.hidden_size // self.num_heads
+        self.max_position_embeddings = config.max_position_embeddings
+        self.num_layers = config.num_hidden_layers
+        self.model_config = config
+
+        self.embedding = Embedding(self.vocab_size, self.hidden_size)
+        self.decoder_layers = nn.ModuleList([DecoderLayer(config, layer_idx=i) for i in range(self.num_layers)])
+        self.final_proj = FinalProjection(self.hidden_size, self.vocab_size, bias=False)
+        RMSNorm = LlamaRMSNorm if os.getenv("FLASH_ATTEN", "1") != "1" else TritonRMSNorm
+        self.final_norm = RMSNorm(self.hidden_size, eps=config.rms_norm_eps)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        # same order as the reference (:279-289) so a seed gives the same weights
+        self.embedding.reset_parameters()
+        for layer in self.decoder_layers:
+            layer.input_layernorm.reset_parameters()
+            layer.attention.reset_parameters()
+            layer.post_attention_layernorm.reset_parameters()
+            layer.mlp.reset_parameters()
+        self.final_norm.reset_parameters()
+        self.final_proj.reset_parameters()
+
+    def set_cp_rank(self, cp_rank: int) -> None:
+        """Re-slice every layer's RoPE tables for another virtual cp rank (the reference builds one model per
+        process, so its slice is fixed at construction, :228)."""
+        mgr = pgm.process_group_manager
+        mgr.set_cp_rank(cp_rank)
+        for layer in self.decoder_layers:
+            head_dim = self.hidden_size // self.num_heads
+            if not hasattr(layer, "_full_tables"):
+                layer._full_tables = get_cos_sin(self.max_position_embeddings, head_dim=head_dim,
+                                                 base=self.model_config.rope_theta)
+            layer.cos, layer.sin = context_parallel.update_rope_for_context_parallel(*layer._full_tables)
+
+    def forward(self, input_ids, attention_mask=None, position_ids: torch.Tensor = None):
+        x = self.embedding(input_ids)
+        for layer in self.decoder_layers:
+            x = layer(x)
+        x = self.final_norm(x)
+        return self.final_proj(x)

@@ -260,13 +260,16 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
     return dk, dv
 
 
-def convert_f32(src: torch.Tensor, dtype, like: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """fp32 contiguous [B,H,S,D] -> dtype, laid out like `like` (same strides) or contiguous."""
+def convert_f32(src: torch.Tensor, dtype, like: Optional[torch.Tensor] = None, bshd: bool = False) -> torch.Tensor:
+    """fp32 contiguous [B,H,S,D] -> dtype; laid out like `like` (same strides), as a view over [B,S,H,D]
+    memory (bshd=True), or contiguous."""
     _dev(src, like)
     if src.dtype != torch.float32 or not src.is_contiguous() or src.dim() != 4:
         raise RuntimeError("convert_f32: src must be a contiguous fp32 [B,H,S,D] tensor")
     B, H, S, D = src.shape
-    if like is not None and _dense(like) and like.stride(-1) == 1:
+    if bshd:
+        dst = empty_bshd(B, H, S, D, dtype, src.device)
+    elif like is not None and _dense(like) and like.stride(-1) == 1:
         dst = torch.empty_strided(src.shape, like.stride(), dtype=dtype, device=src.device)
     else:
         dst = torch.empty(src.shape, dtype=dtype, device=src.device)
