@@ -1,0 +1,304 @@
+"""Benchmark of the hot path on ONE MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Workload (BASELINE.json configs[1]): causal ring attention, q/k/v bf16 [B=4, H=32, S=1024, D=64],
+cp_size = 4 (chunks of 256).  One "step" is forward + backward of the ring for ALL four cp ranks,
+executed one rank after another on the one GPU: rank r attends its 256-query chunk over the K/V
+chunks 0..r (diagonal chunk masked, earlier chunks dense), and its backward adds into the fp32 dK/dV
+accumulators of those chunks.  Each rank's ring steps run fused in one forward and one backward
+launch (the online softmax carries across the chunks; no score matrix or per-chunk partial result
+touches HBM).  The step is recorded once into a HIP graph and replayed K times; inputs are resident
+in HBM before the timed region.
+
+value = algorithmic FLOPs of the step (7 * B*H*S^2*D = 60.13 GFLOP: forward 4 and backward 10 FLOPs
+per (query, key, d) triple, the masked diagonal chunk counted half) / measured time.
+
+The JSON line also carries
+  roofline      the dominant kernel (attention backward) against the dense bf16 MFMA peak,
+  cpu_baseline  the CPU oracle (plain torch restatement of picotron's blockwise ring attention, fp32)
+                timed on this host,
+  extras        forward / backward split, the reference-shaped per-ring-step schedule, and the
+                bandwidth kernels (RMSNorm, RoPE, SwiGLU) against the 8 TB/s HBM peak.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels")
+    return ap.parse_args()
+
+
+class RingBench:
+    """State + one step of the all-ranks ring (fused launches) for configs[1]."""
+
+    def __init__(self, torch, ops, B=4, H=32, S=1024, D=64, W=4, device="cuda"):
+        self.torch, self.ops = torch, ops
+        self.B, self.H, self.S, self.D, self.W = B, H, S, D, W
+        self.Sc = S // W
+        self.scale = 1.0 / math.sqrt(D)
+        g = torch.Generator().manual_seed(0)
+        q = torch.randn(B, H, S, D, generator=g) * self.scale   # "scaled by 1/sqrt(D) on q"
+        k = torch.randn(B, H, S, D, generator=g)
+        v = torch.randn(B, H, S, D, generator=g)
+        do = torch.randn(B, H, S, D, generator=g)
+        self.host = tuple(t.to(torch.bfloat16) for t in (q, k, v, do))
+        self.q, self.k, self.v, self.do = (t.to(device) for t in self.host)
+        f32 = dict(dtype=torch.float32, device=device)
+        self.out = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=device)
+        self.lse = torch.empty(W, B, H, self.Sc, **f32)
+        self.delta = torch.empty(W, B, H, self.Sc, **f32)
+        self.dq_acc = torch.empty(W, B, H, self.Sc, D, **f32)
+        self.dk_acc = torch.empty(B, H, S, D, **f32)
+        self.dv_acc = torch.empty(B, H, S, D, **f32)
+
+    def flops(self):
+        blocks = self.W * (self.W + 1) / 2 - self.W / 2  # diagonal blocks count half
+        per_block = self.B * self.H * self.Sc * self.Sc * self.D
+        return 4 * per_block * blocks, 10 * per_block * blocks
+
+    def _views(self, r):
+        Sc = self.Sc
+        sl_q = slice(r * Sc, (r + 1) * Sc)
+        sl_k = slice(0, (r + 1) * Sc)
+        return (self.q[:, :, sl_q], self.k[:, :, sl_k], self.v[:, :, sl_k], self.do[:, :, sl_q], self.out[:, :, sl_q],
+                self.dk_acc[:, :, sl_k], self.dv_acc[:, :, sl_k])
+
+    def forward(self):
+        for r in range(self.W):
+            q, k, v, _, out, _, _ = self._views(r)
+            self.ops.attn_fwd(q, k, v, self.scale, True, r * self.Sc, out=out, lse=self.lse[r])
+
+    def backward_kernels_only(self):
+        for r in range(self.W):
+            q, k, v, do, out, dk, dv = self._views(r)
+            self.ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, self.dq_acc[r],
+                              dk, dv, accumulate=True)
+
+    def backward(self):
+        self.dk_acc.zero_()
+        self.dv_acc.zero_()
+        ops = self.ops
+        for r in range(self.W):
+            q, k, v, do, out, dk, dv = self._views(r)
+            delta = ops.attn_bwd_preprocess(do, out, self.dq_acc[r], delta=self.delta[r])
+            ops.attn_bwd(do, q, k, v, self.lse[r], delta, self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
+                         accumulate=True)
+        # hand the gradients back in the dtype of the inputs (autograd's cast in the reference)
+        self.dq = [ops.convert_f32(self.dq_acc[r], self.torch.bfloat16) for r in range(self.W)]
+        self.dk = ops.convert_f32(self.dk_acc, self.torch.bfloat16)
+        self.dv = ops.convert_f32(self.dv_acc, self.torch.bfloat16)
+
+    def step(self):
+        self.forward()
+        self.backward()
+
+    # -- the same work in the reference's shape: one launch per ring step (block + fused merge)
+    def step_per_ring_step(self):
+        torch, ops, Sc = self.torch, self.ops, self.Sc
+        self.dk_acc.zero_()
+        self.dv_acc.zero_()
+        for r in range(self.W):
+            q = self.q[:, :, r * Sc:(r + 1) * Sc]
+            do = self.do[:, :, r * Sc:(r + 1) * Sc]
+            out32 = torch.empty(self.B, self.H, Sc, self.D, dtype=torch.float32, device=q.device)
+            lse = self.lse[r]
+            for s in range(r + 1):
+                c = r - s
+                ops.attn_fwd(q, self.k[:, :, c * Sc:(c + 1) * Sc], self.v[:, :, c * Sc:(c + 1) * Sc], self.scale, s == 0, 0,
+                             out=out32, lse=lse, merge=s > 0)
+            out = ops.convert_f32(out32, torch.bfloat16)
+            delta = ops.attn_bwd_preprocess(do, out, self.dq_acc[r])
+            for s in range(r + 1):
+                c = r - s
+                sl = slice(c * Sc, (c + 1) * Sc)
+                ops.attn_bwd(do, q, self.k[:, :, sl], self.v[:, :, sl], lse, delta, self.scale, s == 0, 0, self.dq_acc[r],
+                             self.dk_acc[:, :, sl], self.dv_acc[:, :, sl], accumulate=True)
+        self.dq = [ops.convert_f32(self.dq_acc[r], torch.bfloat16) for r in range(self.W)]
+        self.dk = ops.convert_f32(self.dk_acc, torch.bfloat16)
+        self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
+
+
+def graph_time(torch, fn, iters, warmup=3):
+    """Records fn() once into a HIP graph and returns (ms per replay over `iters` replays, graph)."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(warmup):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    for _ in range(2):
+        graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        graph.replay()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / iters, graph
+
+
+def bandwidth_extras(torch, ops, iters=50):
+    """RMSNorm / RoPE / SwiGLU at the SmolLM-1.7B step's sizes (T = 4096 tokens, h 2048, I 8192, 32 heads of 64).
+    `cold` rotates over enough buffers to exceed the 256 MB Infinity Cache, `warm` reuses one set."""
+    dev = "cuda"
+    bf = torch.bfloat16
+    T, h, I, B, H, S, D = 4096, 2048, 8192, 4, 32, 1024, 64
+    res = {}
+
+    def run(name, make, call, bytes_per_call, nsets_cold):
+        for label, nsets in (("cold", nsets_cold), ("warm", 1)):
+            sets = [make() for _ in range(nsets)]
+            def body():
+                for s_ in sets:
+                    call(*s_)
+            ms, _ = graph_time(torch, body, iters)
+            gbs = bytes_per_call * nsets / (ms * 1e-3) / 1e9
+            res[f"{name}_{label}"] = {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3),
+                                      "us_per_call": round(ms * 1e3 / nsets, 2), "algorithmic_MB": round(bytes_per_call / 1e6, 2)}
+            del sets
+
+    w = torch.ones(h, dtype=bf, device=dev)
+    run("rmsnorm_fwd", lambda: (torch.randn(T, h, device=dev).to(bf),),
+        lambda x: ops.rmsnorm_fwd(x, w, 1e-5, False), 2 * T * h * 2 + h * 2, 24)
+    rstd = torch.rand(T, device=dev) + 0.5
+    run("rmsnorm_bwd", lambda: (torch.randn(T, h, device=dev).to(bf), torch.randn(T, h, device=dev).to(bf)),
+        lambda dy, x: ops.rmsnorm_bwd(dy, x, w, rstd), 3 * T * h * 2 + h * 4, 16)
+    cos = torch.rand(S, D, device=dev).to(bf)
+    sin = torch.rand(S, D, device=dev).to(bf)
+    run("rope", lambda: (torch.randn(B, S, H, D, device=dev).to(bf).transpose(1, 2),),
+        lambda x: ops.rope(x, cos, sin), 2 * B * H * S * D * 2 + S * D * 2, 24)
+    run("swiglu_fwd", lambda: (torch.randn(T, I, device=dev).to(bf), torch.randn(T, I, device=dev).to(bf)),
+        lambda g_, u: ops.swiglu_fwd(g_, u), 3 * T * I * 2, 4)
+    run("swiglu_bwd", lambda: tuple(torch.randn(T, I, device=dev).to(bf) for _ in range(3)),
+        lambda dy, g_, u: ops.swiglu_bwd(dy, g_, u), 5 * T * I * 2, 3)
+    return res
+
+
+def cpu_baseline(host_tensors, W, scale, flops_total):
+    """The CPU oracle on the same inputs: full configs[1] shape, fp32, all host threads and one thread."""
+    import torch
+    from oracle import ring
+    q, k, v, do = (t.float() for t in host_tensors)
+    out = {}
+    cores = min(os.cpu_count() or 1, 16)
+    for label, threads, reps in (("all_threads", cores, 4), ("one_thread", 1, 1)):
+        torch.set_num_threads(threads)
+        ring.all_ranks_forward(q[:1], k[:1], v[:1], W, scale, True)  # warm the allocator
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            o, l = ring.all_ranks_forward(q, k, v, W, scale, True)
+            ring.all_ranks_backward(do, q, k, v, o, l, W, scale, True)
+        dt = (time.perf_counter() - t0) / reps
+        out[label] = {"value": round(flops_total / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "s_per_step": round(dt, 3)}
+    torch.set_num_threads(cores)
+    return out
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU: this build has no multi-GPU path (asked for --gpus {args.gpus}); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from picotron_amd import ops
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    ops._lib.lib()  # fail loudly now if the HIP library is not built
+
+    rb = RingBench(torch, ops)
+    fwd_flops, bwd_flops = rb.flops()
+    total_flops = fwd_flops + bwd_flops
+
+    # ---- warm-up (eager), then the timed K replays of the recorded step
+    for _ in range(max(args.warmup, 1)):
+        rb.step()
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        rb.step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rb.step()
+    graph.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        graph.replay()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    value = total_flops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- dominant kernel: the backward launches alone, HIP events on the launching stream
+    ms_bwd_k, _ = graph_time(torch, rb.backward_kernels_only, max(args.steps // 2, 10))
+    bwd_launch_us = ms_bwd_k * 1e3 / rb.W
+    bwd_tflops = bwd_flops / (ms_bwd_k * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "attn_bwd_kernel<64>", "achieved": round(bwd_tflops, 2),
+                "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(bwd_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                "avg_launch_us": round(bwd_launch_us, 2), "flops_per_launch": bwd_flops / rb.W, "traffic": None}
+
+    extras = {}
+    if not args.no_extras:
+        ms_fwd, _ = graph_time(torch, rb.forward, max(args.steps // 2, 10))
+        extras["attn_fwd"] = {"TFLOP/s": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2), "us_per_launch": round(ms_fwd * 1e3 / rb.W, 2),
+                              "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
+        extras["per_ring_step_schedule"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4)}
+        t0 = time.perf_counter()
+        for _ in range(20):
+            rb.step()
+        torch.cuda.synchronize()
+        extras["eager_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / 20, 4)
+        extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
+
+    line = {
+        "metric": "causal ring-attn fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[1]: causal ring attention fwd+bwd, B4 H32 S1024 D64, cp_size 4, all 4 ranks' ring "
+                               "steps run one rank after another on one GPU (one fused launch per rank and direction)",
+                   "global_batch": 4, "seq_len": 1024, "flops_per_step": total_flops},
+        "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 4),
+        "roofline": roofline,
+    }
+    if not args.no_cpu:
+        cpu = cpu_baseline(rb.host, rb.W, rb.scale, total_flops)
+        main_leg = cpu["all_threads"]
+        line["cpu_baseline"] = {"value": main_leg["value"], "unit": "TFLOP/s", "cores": main_leg["cores"], "kind": "port",
+                                "sample": f"full configs[1] shape (fwd+bwd of all 4 ranks), fp32, {main_leg['s_per_step']} s per step; "
+                                          f"one thread: {cpu['one_thread']['value']} TFLOP/s ({cpu['one_thread']['s_per_step']} s per step)"}
+    if extras:
+        line["extras"] = extras
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -156,13 +156,15 @@ int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* dout, const
  * lse, delta: [B,Hq,Sq] fp32 (lse is the FINAL merged lse, as in the reference).
  * dq_acc: [B,Hq,Sq,D] contiguous fp32, accumulated with atomic adds (zero it first, or keep the
  *         running sum across ring steps).
- * dk, dv: [B,Hkv,Sk,D] contiguous; dkv_dtype PICO_F32 with accumulate = 1 adds into the buffers
- *         (the travelling fp32 accumulators of the ring), accumulate = 0 overwrites; PICO_BF16 overwrites.
+ * dk, dv: [B,Hkv,Sk,D] addressed by dkv_stride (element strides for b, h, s; NULL = contiguous);
+ *         dkv_dtype PICO_F32 with accumulate = 1 adds into the buffers (the travelling fp32 accumulators
+ *         of the ring), accumulate = 0 overwrites; PICO_BF16 overwrites.
  *         With Hq > Hkv the group's query heads are reduced inside the kernel.
  */
 int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
                   const void* dout, const float* lse, const float* delta,
-                  float* dq_acc, void* dk, void* dv, int dkv_dtype, int accumulate, void* stream);
+                  float* dq_acc, void* dk, void* dv, const int64_t* dkv_stride,
+                  int dkv_dtype, int accumulate, void* stream);
 
 /* fp32 -> bf16/fp32 conversion with layout change: src [B,H,S,D] contiguous fp32,
  * dst addressed by dst_stride (b,h,s).  Used to hand dq_acc back in the dtype / layout of q.

@@ -9,9 +9,20 @@
 //   dV += P^T dO,  dK += dS^T Q      (P / dS feed the MFMA straight from registers as the A operand;
 //                                     dO and Q come from the row-major LDS tiles through transposing reads)
 //   dS^T -> LDS, barrier
-//   dQ  = dS K * scale               (16x16x32 MFMA, each wave takes 16 query rows over all 128 keys;
-//                                     both operands through transposing LDS reads) -> fp32 atomic adds
+//   dQ  = dS K * scale               (each wave owns 32x32 blocks of the 64 x D tile over all 128 keys; K
+//                                     fragments stay in registers, dS comes back through transposing
+//                                     LDS reads) -> fp32 atomic adds
 #include "attn_common.h"
+
+#include <type_traits>
+
+#if defined(PICO_BWD_TIMING)
+__device__ long long pico_dbg[64];
+#define PICO_T(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && it == 2) pico_dbg[i] = clock64(); } while (0)
+extern "C" int pico_debug_read(long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(pico_dbg), sizeof(long long) * 64); }
+#else
+#define PICO_T(i)
+#endif
 
 namespace pico {
 namespace {
@@ -26,6 +37,7 @@ struct BwdParams {
   void* dv;
   int dkv_f32;
   int accumulate;
+  int64_t dks[3];  // element strides (b, h, s) of dk and dv
 };
 
 template <int D>
@@ -40,11 +52,11 @@ struct BwdCfg {
   static constexpr int kQLoads = BM * kVecPerRow / kThreads;
   static constexpr int kKLoads = BN * kVecPerRow / kThreads;
   static constexpr size_t kLdsBytes =
-      (2 * BM * LDQ + BN * LDQ + BN * LDS_) * sizeof(__bf16) + 2 * BM * sizeof(float);
+      (2 * BM * LDQ + BN * LDQ + 2 * BN * LDS_) * sizeof(__bf16) + 2 * BM * sizeof(float);
 };
 
 template <int D>
-__global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
+__device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
   using C = BwdCfg<D>;
   constexpr int BM = C::BM, BN = C::BN, LDQ = C::LDQ, LDS_ = C::LDS_;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -52,11 +64,14 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
   __bf16* sdO = sQ + BM * LDQ;
   __bf16* sK = sdO + BM * LDQ;
   __bf16* sdS = sK + BN * LDQ;
-  float* sL = reinterpret_cast<float*>(sdS + BN * LDS_);
+  float* sL = reinterpret_cast<float*>(sdS + 2 * BN * LDS_);  // sdS is double-buffered
   float* sDelta = sL + BM;
 
   const AttnParams& a = p.a;
-  const int ktile = blockIdx.x, hkv = blockIdx.y, b = blockIdx.z;
+  // grid = (Hkv * B, key tiles): the x index runs fastest in dispatch order, so all heads of key tile 0
+  // (the longest under a causal mask) start first and the short tiles fill in behind them; workgroups of
+  // one head are a multiple of 8 apart in dispatch order and so share an XCD's L2
+  const int ktile = blockIdx.y, hkv = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
   const int group = a.Hq / a.Hkv;
   const int key0 = ktile * BN;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -92,6 +107,23 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
     *reinterpret_cast<u32x4*>(&sK[r * LDQ + cv * 8]) = raw;
   }
 
+  // ---- K as the B operand of dQ = dS K (B[k = key][n = d]) for the dQ blocks this wave owns: read
+  //      once through transposing LDS reads and kept in registers
+  constexpr int kDqBlocks = (BM / 32) * (D / 32);
+  constexpr int kDqPasses = kDqBlocks / C::NW;
+  static_assert(kDqBlocks % C::NW == 0, "dQ blocks must split evenly over the waves");
+  bf16x8 ktf[kDqPasses][BN / 16];
+  __syncthreads();
+#pragma unroll
+  for (int pass = 0; pass < kDqPasses; ++pass) {
+    const int db_w = (pass * C::NW + wave) % (D / 32);
+#pragma unroll
+    for (int ks = 0; ks < BN / 16; ++ks) {
+      const int krow = 16 * ks + 4 * h + (lane % 16) / 4;
+      ktf[pass][ks] = lds_read_tr_pair(&sK[krow * LDQ + 32 * db_w + 16 * ((lane / 16) % 2) + 4 * (lane % 4)], LDQ);
+    }
+  }
+
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
 #pragma unroll
   for (int db = 0; db < D / 32; ++db)
@@ -108,8 +140,11 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
   const int tiles_per_head = n_qtiles > qt_start ? n_qtiles - qt_start : 0;
   const int n_iter = tiles_per_head * group;
 
+  // Global -> register prefetch of the next Q / dO tile (+ lse, delta).  Loads are unconditional (rows
+  // past Sq are clamped to the last row and zeroed when they are written to LDS) and nothing here uses a
+  // loaded value, so the loop never has to wait for memory inside the prefetch.
   u32x4 qreg[C::kQLoads], doreg[C::kQLoads];
-  float lreg = INFINITY, dreg = 0.f;
+  float lreg = 0.f, dreg = 0.f;
   auto prefetch = [&](int it) {
     const int hq = hkv * group + it / tiles_per_head;
     const int q0 = (qt_start + it % tiles_per_head) * BM;
@@ -119,50 +154,102 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
     for (int i = 0; i < C::kQLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      u32x4 zq = {0, 0, 0, 0}, zo = {0, 0, 0, 0};
-      if (q0 + r < a.Sq) {
-        zq = *reinterpret_cast<const u32x4*>(qb + static_cast<int64_t>(q0 + r) * a.qs[2] + cv * 8);
-        zo = *reinterpret_cast<const u32x4*>(dob + static_cast<int64_t>(q0 + r) * a.os[2] + cv * 8);
-      }
-      qreg[i] = zq;
-      doreg[i] = zo;
+      const int row = (q0 + r < a.Sq) ? q0 + r : a.Sq - 1;
+      qreg[i] = *reinterpret_cast<const u32x4*>(qb + static_cast<int64_t>(row) * a.qs[2] + cv * 8);
+      doreg[i] = *reinterpret_cast<const u32x4*>(dob + static_cast<int64_t>(row) * a.os[2] + cv * 8);
     }
-    if (tid < BM) {
-      // rows past Sq (and rows whose lse is -inf: they saw no key) get lse = +inf so that P = 0
-      lreg = INFINITY;
-      dreg = 0.f;
-      if (q0 + tid < a.Sq) {
-        const int64_t row = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + q0 + tid;
-        const float l = p.lse[row];
-        lreg = (l == -INFINITY) ? INFINITY : l * kLog2e;
-        dreg = p.delta[row];
-      }
+    {
+      const int r = tid % BM;
+      const int row = (q0 + r < a.Sq) ? q0 + r : a.Sq - 1;
+      const int64_t gi = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + row;
+      lreg = p.lse[gi];
+      dreg = p.delta[gi];
     }
   };
 
   if (n_iter > 0) prefetch(0);
 
-  for (int it = 0; it < n_iter; ++it) {
-    const int hq = hkv * group + it / tiles_per_head;
-    const int q0 = (qt_start + it % tiles_per_head) * BM;
-    __syncthreads();  // previous dQ phase has finished with sdS; previous S phase with sQ / sdO
+  // Software pipeline over the (head, query tile) pairs.  Trip `it` stages tile `it` in LDS and runs its
+  // S phase, and first finishes tile `it - 1`: its dS^T sits in the other half of the double-buffered
+  // sdS, so the dQ product and its atomics are issued a whole trip before anything waits on memory
+  // again, and one barrier per tile disappears.  The prefetch loads are issued after those atomics, so
+  // the wait before the next LDS fill covers operations that have had a full trip to complete.
+  int prev_hq = 0, prev_q0 = 0;
+  for (int it = 0; it <= n_iter; ++it) {
+    const bool have_tile = it < n_iter;
+    const int hq = hkv * group + (have_tile ? it / tiles_per_head : 0);
+    const int q0 = (qt_start + (have_tile ? it % tiles_per_head : 0)) * BM;
+    PICO_T(0);
+    __syncthreads();  // S phase of tile it-1 is complete: sdS[(it-1)&1] is full, sQ / sdO are free
+    PICO_T(1);
+    if (have_tile) {
 #pragma unroll
-    for (int i = 0; i < C::kQLoads; ++i) {
-      const int idx = tid + i * C::kThreads;
-      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = qreg[i];
-      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = doreg[i];
+      for (int i = 0; i < C::kQLoads; ++i) {
+        const int idx = tid + i * C::kThreads;
+        const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+        const bool live = q0 + r < a.Sq;
+        const u32x4 zero = {0, 0, 0, 0};
+        *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = live ? qreg[i] : zero;
+        *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = live ? doreg[i] : zero;
+      }
+      if (tid < BM) {
+        // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
+        const bool live = q0 + tid < a.Sq && lreg != -INFINITY;
+        sL[tid] = live ? lreg * kLog2e : INFINITY;
+        sDelta[tid] = live ? dreg : 0.f;
+      }
     }
-    if (tid < BM) { sL[tid] = lreg; sDelta[tid] = dreg; }
+    PICO_T(2);
     __syncthreads();
+    PICO_T(3);
+
+    // ================= dQ of the previous tile: the 64 x D tile is cut into 32 x 32 blocks, NW per pass
+#if !defined(PICO_BWD_NO_DQ)
+    if (it > 0) {
+      const __bf16* sdS_prev = sdS + ((it - 1) & 1) * (BN * LDS_);
+#pragma unroll
+      for (int pass = 0; pass < kDqPasses; ++pass) {
+        const int blk = pass * C::NW + wave;         // block index: query half x d block
+        const int qb_w = blk / (D / 32), db_w = blk % (D / 32);
+        f32x16 dq;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dq[i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < BN / 16; ++ks) {
+          // A[m = query][k = key]: slots 4jj+t <- keys 16ks + 8jj + 4h + t, read transposed from dS^T[key][query]
+          const int krow = 16 * ks + 4 * h + (lane % 16) / 4;
+          const bf16x8 af = lds_read_tr_pair(&sdS_prev[krow * LDS_ + 32 * qb_w + 16 * ((lane / 16) % 2) + 4 * (lane % 4)], LDS_);
+          dq = mfma32(af, ktf[pass][ks], dq);
+        }
+        // rows past Sq add 0 to the last valid row instead of branching around the atomic
+        float* dqp = p.dq_acc + ((static_cast<int64_t>(b) * a.Hq + prev_hq) * a.Sq) * D + 32 * db_w + n;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const int qrow = prev_q0 + 32 * qb_w + 8 * (i / 4) + 4 * h + (i % 4);
+          const bool live = qrow < a.Sq;
+          const float val = live ? dq[i] * a.sm_scale : 0.f;
+          float* dst = dqp + static_cast<int64_t>(live ? qrow : a.Sq - 1) * D;
+#if defined(PICO_BWD_NO_ATOMIC)
+          *dst = val;
+#else
+          unsafeAtomicAdd(dst, val);
+#endif
+        }
+      }
+    }
+#endif
+    PICO_T(4);
+    if (!have_tile) break;
     if (it + 1 < n_iter) prefetch(it + 1);
+    PICO_T(5);
 
     // ================= S phase: this wave's 32 keys against the tile's 64 queries
+    __bf16* sdS_cur = sdS + (it & 1) * (BN * LDS_);
     const int kw0 = key0 + 32 * wave;
 #pragma unroll
     for (int sb = 0; sb < BM / 32; ++sb) {
       const int qs_pos = a.q_offset + q0 + 32 * sb;  // position of the sub-block's first query
-      __bf16* ds_dst = &sdS[(32 * wave + n) * LDS_ + 32 * sb + 4 * h];
+      __bf16* ds_dst = &sdS_cur[(32 * wave + n) * LDS_ + 32 * sb + 4 * h];
       if (a.causal && kw0 > qs_pos + 31) {  // every (query, key) pair of this 32x32 block is masked
 #pragma unroll
         for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x2*>(ds_dst + 8 * j) = u32x2{0, 0};
@@ -178,21 +265,28 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
         s_acc = mfma32(qa, kf[s], s_acc);
         dp_acc = mfma32(da, vf[s], dp_acc);
       }
-      const bool need_mask = a.causal && (kw0 + 31 > qs_pos);
-      const int key = kw0 + n;
+      // P = exp2(S*c - lse*log2e), dS = P * (dP - delta); the mask test is paid only on the diagonal
+      auto softmax_grad = [&](auto mask_c) {
+        constexpr bool kMask = decltype(mask_c)::value;
+        const int key_rel = kw0 + n - qs_pos - 4 * h;  // key is masked for row (8j + 4h + t) iff key_rel > 8j + t
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
+        for (int j = 0; j < 4; ++j) {
+          const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-          const int i = 4 * j + t;
-          float pv = fast_exp2(s_acc[i] * c - l4[t]);
-          if (need_mask && key > qs_pos + 8 * j + 4 * h + t) pv = 0.f;
-          s_acc[i] = pv;
-          dp_acc[i] = pv * (dp_acc[i] - d4[t]);
+          for (int t = 0; t < 4; ++t) {
+            const int i = 4 * j + t;
+            float pv = fast_exp2(s_acc[i] * c - l4[t]);
+            if constexpr (kMask) {
+              if (key_rel > 8 * j + t) pv = 0.f;
+            }
+            s_acc[i] = pv;
+            dp_acc[i] = pv * (dp_acc[i] - d4[t]);
+          }
         }
-      }
+      };
+      if (a.causal && kw0 + 31 > qs_pos) softmax_grad(std::true_type{});
+      else softmax_grad(std::false_type{});
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
         const bf16x8 pf = pack8(s_acc, 8 * cc);
@@ -212,64 +306,61 @@ __global__ __launch_bounds__(256) void attn_bwd_kernel(const BwdParams p) {
         }
       }
     }
-    __syncthreads();
-
-    // ================= dQ phase: 16 query rows per wave, all 128 keys
-    {
-      const int m16 = lane % 16, g = lane / 16;
-      f32x4 dq[D / 16];
-#pragma unroll
-      for (int nb = 0; nb < D / 16; ++nb) dq[nb] = f32x4{0.f, 0.f, 0.f, 0.f};
-      typedef __attribute__((ext_vector_type(8))) short s16x8;
-#pragma unroll
-      for (int ks = 0; ks < BN / 32; ++ks) {
-        // A[m = query][k = key]: slots e<4 -> keys 32ks + 8g + e, e>=4 -> +4
-        const int krow = 32 * ks + 8 * g + m16 / 4;
-        const __bf16* pa = &sdS[krow * LDS_ + 16 * wave + 4 * (m16 % 4)];
-        const s16x4 a_lo = lds_read_tr(pa);
-        const s16x4 a_hi = lds_read_tr(pa + 4 * LDS_);
-        const bf16x8 af = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(a_lo, a_hi, 0, 1, 2, 3, 4, 5, 6, 7));
-#pragma unroll
-        for (int nb = 0; nb < D / 16; ++nb) {
-          const __bf16* pb = &sK[krow * LDQ + 16 * nb + 4 * (m16 % 4)];
-          const s16x4 b_lo = lds_read_tr(pb);
-          const s16x4 b_hi = lds_read_tr(pb + 4 * LDQ);
-          const bf16x8 bf = __builtin_bit_cast(bf16x8, (s16x8)__builtin_shufflevector(b_lo, b_hi, 0, 1, 2, 3, 4, 5, 6, 7));
-          dq[nb] = mfma16(af, bf, dq[nb]);
-        }
-      }
-      float* dqp = p.dq_acc + ((static_cast<int64_t>(b) * a.Hq + hq) * a.Sq) * D;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int qrow = q0 + 16 * wave + 4 * g + i;
-        if (qrow < a.Sq) {
-#pragma unroll
-          for (int nb = 0; nb < D / 16; ++nb)
-            unsafeAtomicAdd(dqp + static_cast<int64_t>(qrow) * D + 16 * nb + m16, dq[nb][i] * a.sm_scale);
-        }
-      }
-    }
+    PICO_T(6);
+    prev_hq = hq;
+    prev_q0 = q0;
   }
 
-  // ---- epilogue: dK (scaled) and dV rows of this wave's keys
+  // ---- epilogue: dK (scaled) and dV rows of this wave's keys.  In accumulate mode all reads of a block
+  //      are issued before the first write so they overlap instead of serialising on memory latency.
 #pragma unroll
-  for (int db = 0; db < D / 32; ++db)
+  for (int db = 0; db < D / 32; ++db) {
+    int64_t off[16];
+    bool live[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int key = key0 + 32 * wave + 8 * (i / 4) + 4 * h + (i % 4);
-      if (key >= a.Sk) continue;
-      const int64_t off = ((static_cast<int64_t>(b) * a.Hkv + hkv) * a.Sk + key) * D + 32 * db + n;
-      const float vk = dk_acc[db][i] * a.sm_scale, vv = dv_acc[db][i];
-      if (p.dkv_f32) {
-        float* pk = static_cast<float*>(p.dk) + off;
-        float* pv = static_cast<float*>(p.dv) + off;
-        if (p.accumulate) { *pk += vk; *pv += vv; } else { *pk = vk; *pv = vv; }
-      } else {
-        static_cast<__bf16*>(p.dk)[off] = static_cast<__bf16>(vk);
-        static_cast<__bf16*>(p.dv)[off] = static_cast<__bf16>(vv);
-      }
+      live[i] = key < a.Sk;
+      off[i] = b * p.dks[0] + hkv * p.dks[1] + static_cast<int64_t>(live[i] ? key : 0) * p.dks[2] + 32 * db + n;
     }
+    if (p.dkv_f32) {
+      float* pk = static_cast<float*>(p.dk);
+      float* pv = static_cast<float*>(p.dv);
+      float ok[16], ov[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) { ok[i] = 0.f; ov[i] = 0.f; }
+      if (p.accumulate) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+          if (live[i]) { ok[i] = pk[off[i]]; ov[i] = pv[off[i]]; }
+      }
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (live[i]) {
+          pk[off[i]] = ok[i] + dk_acc[db][i] * a.sm_scale;
+          pv[off[i]] = ov[i] + dv_acc[db][i];
+        }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (live[i]) {
+          static_cast<__bf16*>(p.dk)[off[i]] = static_cast<__bf16>(dk_acc[db][i] * a.sm_scale);
+          static_cast<__bf16*>(p.dv)[off[i]] = static_cast<__bf16>(dv_acc[db][i]);
+        }
+    }
+  }
 }
+
+// D = 64 fits two workgroups per CU (<= 256 registers per lane), which lets one workgroup's MFMA
+// work overlap the other's softmax / LDS phases; D = 128 needs the full register file.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_kernel_d64(const BwdParams p) {
+  attn_bwd_body<64>(p);
+}
+__global__ __launch_bounds__(256) void attn_bwd_kernel_d128(const BwdParams p) { attn_bwd_body<128>(p); }
+
+template <int D> struct BwdKernel;
+template <> struct BwdKernel<64> { static constexpr auto fn = &attn_bwd_kernel_d64; };
+template <> struct BwdKernel<128> { static constexpr auto fn = &attn_bwd_kernel_d128; };
 
 // delta[row] = sum_d dO * O, one 16-byte vector of each per lane, D/8 lanes per row.
 template <int D, typename TO>
@@ -319,13 +410,13 @@ int launch_bwd(const BwdParams& p, hipStream_t s) {
   using C = BwdCfg<D>;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_bwd_kernel<D>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(BwdKernel<D>::fn),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(C::kLdsBytes)) != hipSuccess)
       return fail(PICO_ERR_LAUNCH, "pico_attn_bwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
     attr_set = true;
   }
   const int n_ktiles = (p.a.Sk + C::BN - 1) / C::BN;
-  hipLaunchKernelGGL((attn_bwd_kernel<D>), dim3(n_ktiles, p.a.Hkv, p.a.B), dim3(C::kThreads), C::kLdsBytes, s, p);
+  hipLaunchKernelGGL(BwdKernel<D>::fn, dim3(p.a.Hkv * p.a.B, n_ktiles), dim3(C::kThreads), C::kLdsBytes, s, p);
   return PICO_OK;
 }
 
@@ -359,8 +450,8 @@ extern "C" int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* 
 }
 
 extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
-                             const float* lse, const float* delta, float* dq_acc, void* dk, void* dv, int dkv_dtype,
-                             int accumulate, void* stream) {
+                             const float* lse, const float* delta, float* dq_acc, void* dk, void* dv,
+                             const int64_t* dkv_stride, int dkv_dtype, int accumulate, void* stream) {
   if (int rc = check_attn_desc("pico_attn_bwd", desc)) return rc;
   if (dkv_dtype != PICO_BF16 && dkv_dtype != PICO_F32)
     return fail(PICO_ERR_DTYPE, "pico_attn_bwd: dk/dv dtype code %d not supported", dkv_dtype);
@@ -376,6 +467,16 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
   p.lse = lse; p.delta = delta; p.dq_acc = dq_acc; p.dk = dk; p.dv = dv;
   p.dkv_f32 = dkv_dtype == PICO_F32;
   p.accumulate = accumulate != 0;
+  if (dkv_stride) {
+    for (int i = 0; i < 3; ++i) {
+      if (dkv_stride[i] < 0) return fail(PICO_ERR_STRIDE, "pico_attn_bwd: negative dk/dv stride");
+      p.dks[i] = dkv_stride[i];
+    }
+  } else {
+    p.dks[2] = desc->D;
+    p.dks[1] = static_cast<int64_t>(desc->Sk) * desc->D;
+    p.dks[0] = p.dks[1] * desc->Hkv;
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   int rc = desc->D == 64 ? launch_bwd<64>(p, s) : launch_bwd<128>(p, s);
   if (rc) return rc;

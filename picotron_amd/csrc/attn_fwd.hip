@@ -40,8 +40,10 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(const FwdParams p) {
 
   const AttnParams& a = p.a;
   const int n_qtiles = (a.Sq + BM - 1) / BM;
-  const int qtile = n_qtiles - 1 - static_cast<int>(blockIdx.x);  // causal: longest tiles first
-  const int hq = blockIdx.y, b = blockIdx.z;
+  // grid = (Hq * B, query tiles): x runs fastest in dispatch order, so every head's last query tile (the
+  // longest under a causal mask) starts first and the short tiles fill in behind
+  const int qtile = n_qtiles - 1 - static_cast<int>(blockIdx.y);
+  const int hq = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
   const int hkv = hq / (a.Hq / a.Hkv);
   const int q0 = qtile * BM;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -252,7 +254,7 @@ template <int D, int QB, int NW>
 void launch(const FwdParams& p, hipStream_t s) {
   using C = FwdCfg<D, QB, NW>;
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
-  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW>), dim3(n_qtiles, p.a.Hq, p.a.B), dim3(C::kThreads), 0, s, p);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), 0, s, p);
 }
 
 }  // namespace
@@ -263,7 +265,7 @@ int check_attn_desc(const char* fn, const pico_attn_desc* d) {
   if (d->B < 0 || d->Hq <= 0 || d->Hkv <= 0 || d->Sq < 0 || d->Sk < 0)
     return fail(PICO_ERR_SHAPE, "%s: negative size (B=%d Hq=%d Hkv=%d Sq=%d Sk=%d)", fn, d->B, d->Hq, d->Hkv, d->Sq, d->Sk);
   if (d->Hq % d->Hkv != 0) return fail(PICO_ERR_SHAPE, "%s: Hq=%d is not a multiple of Hkv=%d", fn, d->Hq, d->Hkv);
-  if (d->B > 65535 || d->Hq > 65535) return fail(PICO_ERR_SHAPE, "%s: B and Hq must be <= 65535", fn);
+  if (static_cast<int64_t>(d->B) * d->Hq > 0x7fffffffLL) return fail(PICO_ERR_SHAPE, "%s: B * Hq too large", fn);
   if (d->q_offset < 0) return fail(PICO_ERR_SHAPE, "%s: q_offset=%d must be >= 0", fn, d->q_offset);
   if (!(d->sm_scale > 0.f)) return fail(PICO_ERR_SHAPE, "%s: sm_scale must be positive", fn);
   const int64_t* all[4] = {d->q_stride, d->k_stride, d->v_stride, d->o_stride};
@@ -311,7 +313,16 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
   p.out_f32 = out_dtype == PICO_F32;
   p.merge = merge != 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (desc->D == 64) launch<64, 1, 4>(p, s);
-  else launch<128, 1, 4>(p, s);
+  // Tile choice for D = 64: more waves per workgroup share each staged K/V tile (fewer barriers and
+  // global loads per MFMA), but the launch still has to fill 256 CUs, so small problems get small tiles.
+  if (desc->D == 64) {
+    const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
+    auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
+    if (groups(256) >= 512) launch<64, 1, 8>(p, s);
+    else if (groups(128) >= 512) launch<64, 1, 4>(p, s);
+    else launch<64, 1, 2>(p, s);
+  } else {
+    launch<128, 1, 4>(p, s);
+  }
   return check_launch("pico_attn_fwd");
 }

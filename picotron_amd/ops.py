@@ -214,14 +214,18 @@ def attn_fwd(q, k, v, sm_scale: float, causal: bool, q_offset: int = 0, out: Opt
     return out, lse
 
 
-def attn_bwd_preprocess(dout: torch.Tensor, out: torch.Tensor, dq_acc: Optional[torch.Tensor] = None) -> torch.Tensor:
+def attn_bwd_preprocess(dout: torch.Tensor, out: torch.Tensor, dq_acc: Optional[torch.Tensor] = None,
+                        delta: Optional[torch.Tensor] = None) -> torch.Tensor:
     """delta = sum(dout * out, -1) as fp32 [B,H,S]; zeroes dq_acc (fp32 contiguous [B,H,S,D]) if given."""
     _dev(dout, out, dq_acc)
     dout = _attn_in(dout, "dout")
     if out.stride() != dout.stride():
         out = _like_strided(out, dout)
     B, H, S, D = dout.shape
-    delta = torch.empty(B, H, S, dtype=torch.float32, device=dout.device)
+    if delta is None:
+        delta = torch.empty(B, H, S, dtype=torch.float32, device=dout.device)
+    elif not (delta.is_contiguous() and delta.dtype == torch.float32 and delta.numel() == B * H * S):
+        raise RuntimeError("attn_bwd_preprocess: delta must be contiguous fp32 [B,H,S]")
     d = _desc(dout, dout, dout, dout, 1.0, False, 0)
     if dq_acc is not None and not (dq_acc.is_contiguous() and dq_acc.dtype == torch.float32):
         raise RuntimeError("attn_bwd_preprocess: dq_acc must be contiguous fp32")
@@ -249,13 +253,14 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
         dv = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
         if accumulate:
             raise RuntimeError("attn_bwd: accumulate=True needs existing dk / dv")
-    if not (dk.is_contiguous() and dv.is_contiguous() and dq_acc.is_contiguous()) or dk.dtype != dv.dtype:
-        raise RuntimeError("attn_bwd: dq_acc, dk and dv must be contiguous")
+    if not dq_acc.is_contiguous() or dk.dtype != dv.dtype or dk.stride() != dv.stride() or dk.stride(-1) != 1:
+        raise RuntimeError("attn_bwd: dq_acc must be contiguous; dk and dv must share dtype and strides (unit D stride)")
     if dq_acc.dtype != torch.float32 or lse.dtype != torch.float32 or delta.dtype != torch.float32:
         raise RuntimeError("attn_bwd: dq_acc, lse and delta must be fp32")
     d = _desc(q, k, v, dout, sm_scale, causal, q_offset)
+    dks = (ctypes.c_int64 * 3)(dk.stride(0), dk.stride(1), dk.stride(2))
     check(_lib.lib().pico_attn_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(lse.contiguous()),
-                                   _ptr(delta.contiguous()), _ptr(dq_acc), _ptr(dk), _ptr(dv), _dt(dk, "dk/dv"),
+                                   _ptr(delta.contiguous()), _ptr(dq_acc), _ptr(dk), _ptr(dv), dks, _dt(dk, "dk/dv"),
                                    int(accumulate), _stream()))
     return dk, dv
 
