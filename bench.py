@@ -3,12 +3,14 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 Workload (BASELINE.json configs[1]): causal ring attention, q/k/v bf16 [B=4, H=32, S=1024, D=64],
-cp_size = 4 (chunks of 256).  One "step" is forward + backward of the ring for ALL four cp ranks,
-executed one rank after another on the one GPU: rank r attends its 256-query chunk over the K/V
-chunks 0..r (diagonal chunk masked, earlier chunks dense), and its backward adds into the fp32 dK/dV
-accumulators of those chunks.  Each rank's ring steps run fused in one forward and one backward
-launch (the online softmax carries across the chunks; no score matrix or per-chunk partial result
-touches HBM).  The step is recorded once into a HIP graph and replayed K times; inputs are resident
+cp_size = 4 (chunks of 256).  One "step" is forward + backward of the ring for ALL four cp ranks on the
+one GPU: rank r attends its 256-query chunk over the K/V chunks 0..r (diagonal chunk masked, earlier
+chunks dense) and its backward adds into dK/dV of those chunks.  The four ranks are batched into one
+launch per direction: the grid's query-tile index enumerates (rank, tile of the rank's chunk), every
+workgroup walks the chunks its rank would receive, the online softmax carries across them (no score
+matrix, no per-chunk partial result and no separate merge pass touches HBM), and dK/dV of a chunk are
+summed over the ranks inside the kernel.  Launches per step: forward, delta pre-pass, backward,
+dq fp32 -> bf16.  The step is recorded once into a HIP graph and replayed K times; inputs are resident
 in HBM before the timed region.
 
 value = algorithmic FLOPs of the step (7 * B*H*S^2*D = 60.13 GFLOP: forward 4 and backward 10 FLOPs
@@ -18,8 +20,9 @@ The JSON line also carries
   roofline      the dominant kernel (attention backward) against the dense bf16 MFMA peak,
   cpu_baseline  the CPU oracle (plain torch restatement of picotron's blockwise ring attention, fp32)
                 timed on this host,
-  extras        forward / backward split, the reference-shaped per-ring-step schedule, and the
-                bandwidth kernels (RMSNorm, RoPE, SwiGLU) against the 8 TB/s HBM peak.
+  extras        forward / backward split; the same step as one launch per rank and as one launch per
+                ring step (the reference's schedule); the bandwidth kernels (RMSNorm, RoPE, SwiGLU)
+                against the 8 TB/s HBM peak; a SmolLM-1.7B-shaped training step (tokens/s).
 """
 from __future__ import annotations
 
@@ -45,6 +48,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels")
+    ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B-shaped training step")
     return ap.parse_args()
 
 
@@ -70,6 +74,11 @@ class RingBench:
         self.dq_acc = torch.empty(W, B, H, self.Sc, D, **f32)
         self.dk_acc = torch.empty(B, H, S, D, **f32)
         self.dv_acc = torch.empty(B, H, S, D, **f32)
+        self.lse_b = torch.empty(B, H, S, **f32)
+        self.delta_b = torch.empty(B, H, S, **f32)
+        self.dq_b = torch.empty(B, H, S, D, **f32)
+        self.dk_b = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=device)
+        self.dv_b = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=device)
 
     def flops(self):
         blocks = self.W * (self.W + 1) / 2 - self.W / 2  # diagonal blocks count half
@@ -111,6 +120,21 @@ class RingBench:
     def step(self):
         self.forward()
         self.backward()
+
+    # -- all four ranks in one launch per direction (q_offset 0 over the whole sequence)
+    def forward_batched(self):
+        self.ops.attn_fwd(self.q, self.k, self.v, self.scale, True, 0, out=self.out, lse=self.lse_b)
+
+    def backward_kernel_batched(self):
+        self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, self.dq_b,
+                          self.dk_b, self.dv_b)
+
+    def step_batched(self):
+        ops = self.ops
+        self.forward_batched()
+        ops.attn_bwd_preprocess(self.do, self.out, self.dq_b, delta=self.delta_b)
+        self.backward_kernel_batched()
+        self.dq_bf16 = ops.convert_f32(self.dq_b, self.torch.bfloat16)
 
     # -- the same work in the reference's shape: one launch per ring step (block + fused merge)
     def step_per_ring_step(self):
@@ -199,6 +223,63 @@ def bandwidth_extras(torch, ops, iters=50):
     return res
 
 
+def train_step_extra(torch, steps=8, warmup=3):
+    """configs[2]: SmolLM-1.7B-shaped training step (24 layers, h 2048, 32 heads, I 8192, V 49152), mbs 4,
+    seq 1024, bf16 parameters with fp32 AdamW master weights and moments, random init, synthetic tokens."""
+    import torch.nn.functional as F
+
+    import picotron_amd.process_group_manager as pgm
+    from oracle.model import smollm_1p7b, synthetic_batch
+    from picotron_amd.model import Llama
+    from picotron_amd.utils import MI355X_BF16_DENSE_FLOPS, flops_per_token, get_num_params
+
+    pgm.setup_process_group_manager(1, 1, 1, 1)
+    os.environ["CONTEXT_PARALLEL"] = "0"
+    cfg = smollm_1p7b(1024)
+    torch.manual_seed(42)
+    with torch.device("cuda"):
+        model = Llama(cfg)
+    model = model.to(torch.bfloat16)
+    params = [p for p in model.parameters()]
+    master = [p.detach().float().clone() for p in params]
+    for m in master:
+        m.grad = torch.zeros_like(m)
+    opt = torch.optim.AdamW(master, lr=3e-4, fused=True)
+    ids, tgt = synthetic_batch(cfg.vocab_size, 4, 1024, seed=0)
+    ids, tgt = ids.cuda(), tgt.cuda()
+
+    def step():
+        for p in params:
+            p.grad = None
+        logits = model(input_ids=ids)
+        loss = F.cross_entropy(logits.view(4 * 1024, -1).float(), tgt.reshape(-1), reduction="mean")
+        loss.backward()
+        with torch.no_grad():
+            torch._foreach_copy_([m.grad for m in master], [p.grad for p in params])
+        opt.step()
+        with torch.no_grad():
+            torch._foreach_copy_([p.data for p in params], master)
+        return loss
+
+    for _ in range(warmup):
+        loss = step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    n = get_num_params(model)
+    tok_s = 4 * 1024 / dt
+    fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, 1024)
+    res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
+           "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
+           "note": "attention / RMSNorm / RoPE / SwiGLU on the HIP kernels; projections, CE and AdamW on torch"}
+    del model, params, master, opt
+    torch.cuda.empty_cache()
+    return res
+
+
 def cpu_baseline(host_tensors, W, scale, flops_total):
     """The CPU oracle on the same inputs: full configs[1] shape, fp32, all host threads and one thread."""
     import torch
@@ -236,17 +317,17 @@ def main():
 
     # ---- warm-up (eager), then the timed K replays of the recorded step
     for _ in range(max(args.warmup, 1)):
-        rb.step()
+        rb.step_batched()
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
-        rb.step()
+        rb.step_batched()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        rb.step()
+        rb.step_batched()
     graph.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -257,34 +338,37 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = total_flops / (ms_per_step * 1e-3) / 1e12
 
-    # ---- dominant kernel: the backward launches alone, HIP events on the launching stream
-    ms_bwd_k, _ = graph_time(torch, rb.backward_kernels_only, max(args.steps // 2, 10))
-    bwd_launch_us = ms_bwd_k * 1e3 / rb.W
+    # ---- dominant kernel: the backward launch alone, HIP events on the launching stream
+    ms_bwd_k, _ = graph_time(torch, rb.backward_kernel_batched, max(args.steps // 2, 10))
     bwd_tflops = bwd_flops / (ms_bwd_k * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "attn_bwd_kernel<64>", "achieved": round(bwd_tflops, 2),
+    roofline = {"bound": "mfma", "kernel": "attn_bwd_kernel_d64", "achieved": round(bwd_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(bwd_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-                "avg_launch_us": round(bwd_launch_us, 2), "flops_per_launch": bwd_flops / rb.W, "traffic": None}
+                "avg_launch_us": round(ms_bwd_k * 1e3, 2), "flops_per_launch": bwd_flops, "traffic": None}
 
     extras = {}
     if not args.no_extras:
-        ms_fwd, _ = graph_time(torch, rb.forward, max(args.steps // 2, 10))
-        extras["attn_fwd"] = {"TFLOP/s": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2), "us_per_launch": round(ms_fwd * 1e3 / rb.W, 2),
-                              "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        ms_fwd, _ = graph_time(torch, rb.forward_batched, max(args.steps // 2, 10))
+        extras["attn_fwd_kernel"] = {"TFLOP/s": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2), "us_per_launch": round(ms_fwd * 1e3, 2),
+                                     "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        ms_rank, _ = graph_time(torch, rb.step, max(args.steps // 4, 10))
+        extras["one_launch_per_rank"] = {"TFLOP/s": round(total_flops / (ms_rank * 1e-3) / 1e12, 2), "ms_per_step": round(ms_rank, 4)}
         ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
-        extras["per_ring_step_schedule"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4)}
+        extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4)}
         t0 = time.perf_counter()
         for _ in range(20):
-            rb.step()
+            rb.step_batched()
         torch.cuda.synchronize()
         extras["eager_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / 20, 4)
         extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
+        if not args.no_train:
+            extras["smollm_1p7b_train_step"] = train_step_extra(torch)
 
     line = {
         "metric": "causal ring-attn fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "configs[1]: causal ring attention fwd+bwd, B4 H32 S1024 D64, cp_size 4, all 4 ranks' ring "
-                               "steps run one rank after another on one GPU (one fused launch per rank and direction)",
+        "config": {"workload": "configs[1]: causal ring attention fwd+bwd, B4 H32 S1024 D64, cp_size 4, the ring steps of all "
+                               "4 ranks on one GPU (ranks batched into one launch per direction)",
                    "global_batch": 4, "seq_len": 1024, "flops_per_step": total_flops},
         "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": roofline,

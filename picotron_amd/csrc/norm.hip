@@ -8,8 +8,8 @@ namespace {
 
 constexpr int kFwdThreads = 256;
 constexpr int kBwdThreads = 512;
-constexpr int kMaxBwdBlocks = 256;   // rows of the dweight workspace
-constexpr int kReduceSlices = 16;
+constexpr int kMaxBwdBlocks = 512;   // rows of the dweight workspace
+constexpr int kBwdWaveThreads = 256; // block size of the row-per-wave backward
 
 template <int G>
 __device__ __forceinline__ float group_sum(float v, float* smem /* this group's 4 floats, G == 256 only */) {
@@ -168,22 +168,147 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
   }
 }
 
-// dweight[c] = sum_p partial[p][c]; 64 columns x 16 slices per block.
-__global__ __launch_bounds__(64 * kReduceSlices) void rmsnorm_dw_reduce_kernel(
+// Row-per-wave backward (hidden <= 64 * NV vectors): a wave keeps the packed x / dy of its row in
+// registers, prefetches the next row while it reduces the current one, and carries its share of
+// dweight in registers across all its rows.  The block's four waves are summed through LDS once at
+// the end and the block writes one row of the partial-sum workspace.
+template <typename T, int NV>
+__global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
+    const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ rstd, T* __restrict__ dx, float* __restrict__ partial,
+    int64_t rows, int hidden) {
+  constexpr int V = io<T>::kVec;
+  constexpr int NWAVE = kBwdWaveThreads / kWave;
+  extern __shared__ float red[];  // [NWAVE - 1][hidden]
+  const int wave = threadIdx.x / kWave, t = threadIdx.x % kWave;
+  const int nvec = hidden / V;
+  const float inv_h = 1.f / static_cast<float>(hidden);
+  float dw[NV][V], wv[NV][V];
+  u32x4 xr[2][NV], dr[2][NV];
+  float rs[2];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+#pragma unroll
+    for (int e = 0; e < V; ++e) { dw[j][e] = 0.f; wv[j][e] = 0.f; }
+    if (t + j * kWave < nvec) io<T>::load(w + (t + j * kWave) * V, wv[j]);
+  }
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * NWAVE;
+  int64_t row = static_cast<int64_t>(blockIdx.x) * NWAVE + wave;
+  auto fetch = [&](int buf, int64_t r) {
+    const int64_t rc = r < rows ? r : rows - 1;  // clamped: the values of a dead row are never used
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * kWave;
+      const int vc = v < nvec ? v : 0;
+      xr[buf][j] = *reinterpret_cast<const u32x4*>(x + rc * hidden + vc * V);
+      dr[buf][j] = *reinterpret_cast<const u32x4*>(dy + rc * hidden + vc * V);
+    }
+    rs[buf] = rstd[rc];
+  };
+  auto unpack = [&](const u32x4& raw, float (&out)[V]) {
+    if constexpr (V == 8) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        out[2 * i] = __uint_as_float(raw[i] << 16);
+        out[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) out[i] = __uint_as_float(raw[i]);
+    }
+  };
+  fetch(0, row);
+  int cur = 0;
+  for (; row < rows; row += stride, cur ^= 1) {
+    fetch(cur ^ 1, row + stride);
+    const float r = rs[cur];
+    float c = 0.f;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      if (t + j * kWave < nvec) {
+        float xv[V], dv[V];
+        unpack(xr[cur][j], xv);
+        unpack(dr[cur][j], dv);
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          const float xh = xv[e] * r;
+          c += dv[e] * wv[j][e] * xh;
+          dw[j][e] += dv[e] * xh;
+        }
+      }
+    }
+    c = wave_sum(c) * inv_h;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * kWave;
+      if (v < nvec) {
+        float xv[V], dv[V], o[V];
+        unpack(xr[cur][j], xv);
+        unpack(dr[cur][j], dv);
+#pragma unroll
+        for (int e = 0; e < V; ++e) o[e] = r * (dv[e] * wv[j][e] - xv[e] * r * c);
+        io<T>::store(dx + row * hidden + v * V, o);
+      }
+    }
+  }
+  // block reduction of dweight: waves 1.. park their share in LDS, wave 0 adds and writes the partial row
+  if (wave > 0) {
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * kWave;
+      if (v < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) red[(wave - 1) * hidden + v * V + e] = dw[j][e];
+      }
+    }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    float* out = partial + static_cast<int64_t>(blockIdx.x) * hidden;
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int v = t + j * kWave;
+      if (v < nvec) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          float acc = dw[j][e];
+#pragma unroll
+          for (int k = 0; k < NWAVE - 1; ++k) acc += red[k * hidden + v * V + e];
+          out[v * V + e] = acc;
+        }
+      }
+    }
+  }
+}
+
+// dweight[c] = sum_p partial[p][c]; 32 columns x 32 slices per block, every thread's loads issued together.
+constexpr int kReduceCols = 32;
+__global__ __launch_bounds__(kReduceCols * 32) void rmsnorm_dw_reduce_kernel(
     const float* __restrict__ partial, float* __restrict__ dweight, int nparts, int hidden) {
-  __shared__ float red[kReduceSlices][64];
-  const int col = blockIdx.x * 64 + threadIdx.x % 64;
-  const int slice = threadIdx.x / 64;
+  constexpr int kSlices = 32, kUnroll = 16;
+  __shared__ float red[kSlices][kReduceCols + 1];
+  const int c = threadIdx.x % kReduceCols;
+  const int col = blockIdx.x * kReduceCols + c;
+  const int slice = threadIdx.x / kReduceCols;
   float s = 0.f;
   if (col < hidden) {
-    for (int p = slice; p < nparts; p += kReduceSlices) s += partial[static_cast<int64_t>(p) * hidden + col];
+    for (int p0 = slice; p0 < nparts; p0 += kSlices * kUnroll) {
+      float v[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const int p = p0 + u * kSlices;
+        v[u] = p < nparts ? partial[static_cast<int64_t>(p) * hidden + col] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) s += v[u];
+    }
   }
-  red[slice][threadIdx.x % 64] = s;
+  red[slice][c] = s;
   __syncthreads();
   if (slice == 0 && col < hidden) {
     float tot = 0.f;
 #pragma unroll
-    for (int i = 0; i < kReduceSlices; ++i) tot += red[i][threadIdx.x];
+    for (int i = 0; i < kSlices; ++i) tot += red[i][c];
     dweight[col] = tot;
   }
 }
@@ -256,6 +381,24 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
     launch_bwd<T, G, NV>(dy, x, w, rstd, dx, partial, blocks, rows, hidden, s);    \
     return PICO_OK;                                                                \
   }
+#define PICO_BWD_WAVE(NV)                                                                              \
+  {                                                                                                    \
+    const int blocks = bwd_blocks(rows, kBwdWaveThreads / kWave);                                      \
+    *blocks_out = blocks;                                                                              \
+    const size_t lds = static_cast<size_t>(kBwdWaveThreads / kWave - 1) * hidden * sizeof(float);      \
+    hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV>), dim3(blocks), dim3(kBwdWaveThreads), lds, s,  \
+                       static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w),  \
+                       rstd, static_cast<T*>(dx), partial, rows, hidden);                              \
+    return PICO_OK;                                                                                    \
+  }
+  if (nv_wave && static_cast<size_t>(hidden) * 3 * sizeof(float) <= 65536) {
+    switch (nv_wave) {
+      case 1: PICO_BWD_WAVE(1);
+      case 2: PICO_BWD_WAVE(2);
+      case 4: PICO_BWD_WAVE(4);
+      default: PICO_BWD_WAVE(8);
+    }
+  }
   if (nv_wave) {
     switch (nv_wave) {
       case 1: PICO_BWD(64, 1);
@@ -269,6 +412,7 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
     case 8: PICO_BWD(256, 8);
     default: break;
   }
+#undef PICO_BWD_WAVE
 #undef PICO_BWD
   return fail(PICO_ERR_SHAPE, "pico_rmsnorm_bwd: hidden=%d too large", hidden);
 }
@@ -317,8 +461,8 @@ extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weigh
   if (!dweight) return fail(PICO_ERR_NULL, "pico_rmsnorm_bwd: dweight is required");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (rows == 0) {  // empty sum: dweight = 0 (the reduce kernel with no partials writes zeros)
-    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + 63) / 64)),
-                       dim3(64 * kReduceSlices), 0, s, static_cast<const float*>(nullptr), dweight, 0,
+    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)),
+                       dim3(kReduceCols * 32), 0, s, static_cast<const float*>(nullptr), dweight, 0,
                        static_cast<int>(hidden));
     return check_launch("pico_rmsnorm_bwd(empty)");
   }
@@ -337,7 +481,7 @@ extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weigh
                : dispatch_bwd<float>(dy, x, weight, rstd, dx, partial, rows, static_cast<int>(hidden), s, &blocks);
   if (rc) return rc;
   if (int lrc = check_launch("pico_rmsnorm_bwd")) return lrc;
-  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + 63) / 64)),
-                     dim3(64 * kReduceSlices), 0, s, partial, dweight, blocks, static_cast<int>(hidden));
+  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)),
+                     dim3(kReduceCols * 32), 0, s, partial, dweight, blocks, static_cast<int>(hidden));
   return check_launch("pico_rmsnorm_bwd(dweight reduce)");
 }

@@ -1,0 +1,101 @@
+"""The C-ABI library loads on a machine without a GPU and exports every symbol include/picotron_amd.h declares.
+Also the host-side logic that needs no GPU: schedule bookkeeping of the local ring and error behaviour."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "picotron_amd.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pico_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for must in ("pico_attn_fwd", "pico_attn_bwd", "pico_attn_bwd_preprocess", "pico_lse_merge", "pico_rmsnorm_fwd",
+                 "pico_rmsnorm_bwd", "pico_rope", "pico_swiglu_fwd", "pico_swiglu_bwd", "pico_version", "pico_last_error"):
+        assert must in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from picotron_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built here (python -m picotron_amd.build)")
+    handle = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(handle, name), f"{name} declared in the header but not exported"
+    assert set(_lib.SIGNATURES) == set(declared_symbols())
+    lib = _lib.lib()
+    assert lib.pico_version().decode().startswith("picotron_amd")
+
+
+def test_argument_checks_run_without_a_gpu():
+    """Validation happens before any launch, so bad arguments are reported even with no device."""
+    from picotron_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built here")
+    lib = _lib.lib()
+    assert lib.pico_rmsnorm_fwd(None, None, None, None, None, None, 4, 7, 1e-5, 1, _lib.PICO_BF16, None) == -3
+    assert b"hidden" in lib.pico_last_error()
+    assert lib.pico_swiglu_fwd(None, None, None, 4, 8, 8, 8, 8, 99, None) == -2
+    d = _lib.AttnDesc()
+    d.B, d.Hq, d.Hkv, d.Sq, d.Sk, d.D, d.sm_scale = 1, 3, 2, 8, 8, 64, 0.125
+    assert lib.pico_attn_fwd(ctypes.byref(d), None, None, None, None, None, 0, 0, None) == -3   # Hq % Hkv != 0
+    d.Hkv, d.D = 3, 96
+    assert lib.pico_attn_fwd(ctypes.byref(d), None, None, None, None, None, 0, 0, None) == -3   # head_dim
+    assert b"head_dim" in lib.pico_last_error()
+    assert lib.pico_rmsnorm_bwd_workspace_bytes(4096, 2048) == 512 * 2048 * 4
+
+
+def test_cpu_tensors_are_refused_not_computed():
+    from picotron_amd import ops
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.rmsnorm_fwd(torch.zeros(2, 8), torch.ones(8), 1e-5, True)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.attn_fwd(*(torch.zeros(1, 1, 8, 64, dtype=torch.bfloat16) for _ in range(3)), 0.125, True)
+
+
+def test_process_group_manager_stand_in():
+    import picotron_amd.process_group_manager as pgm
+    mgr = pgm.setup_process_group_manager(1, 4, 1, 1, cp_rank=2)
+    assert (mgr.cp_rank, mgr.cp_world_size, mgr.cp_send_rank, mgr.cp_recv_rank) == (2, 4, 3, 1)
+    assert mgr.tp_world_size == mgr.pp_world_size == mgr.dp_world_size == 1
+    mgr.set_cp_rank(0)
+    assert (mgr.cp_send_rank, mgr.cp_recv_rank) == (1, 3)          # ring neighbours wrap around
+    with pytest.raises(AssertionError):
+        pgm.setup_process_group_manager(2, 1, 1, 1)                # only cp may exceed 1 on one GPU
+    pgm.setup_process_group_manager(1, 1, 1, 1)
+
+
+def test_local_ring_kv_and_grad_mailbox_on_cpu():
+    """The mailbox protocol itself is host logic: replay two virtual ranks with CPU tensors."""
+    import picotron_amd.process_group_manager as pgm
+    from picotron_amd.context_parallel.cp_communications import ContextCommunicate
+    mgr = pgm.setup_process_group_manager(1, 2, 1, 1)
+    k0, k1 = torch.full((2,), 10.0), torch.full((2,), 11.0)
+    mgr.cp_ring.publish_kv(0, 0, k0, k0)
+    mgr.cp_ring.publish_kv(0, 1, k1, k1)
+    c = ContextCommunicate("comm", rank=1, slot=0)
+    got = c.send_recv(k1)
+    c.commit()
+    c.wait()
+    assert torch.equal(got, k0)                                    # rank 1 receives rank 0's chunk at step 0
+    # gradients: rank 1 first (descending), then rank 0; chunk 0's accumulator must end as the sum
+    g1 = ContextCommunicate("d_kv_comm", rank=1, slot=0)
+    a = g1.send_recv(torch.full((2,), 1.0)); g1.commit(); g1.wait()            # step 0: sends chunk 1, receives chunk 0 (empty)
+    assert torch.equal(a, torch.zeros(2))
+    b = g1.send_recv(a + 5.0); g1.commit(); g1.wait()                          # step 1: sends chunk 0 (+5), receives chunk 1
+    assert torch.equal(b, torch.full((2,), 1.0))
+    g0 = ContextCommunicate("d_kv_comm", rank=0, slot=0)
+    a = g0.send_recv(torch.full((2,), 7.0)); g0.commit(); g0.wait()            # step 0: fresh chunk 0 meets rank 1's 5
+    b = g0.send_recv(a); g0.commit(); g0.wait()                                # step 1: pass-through of chunk 1; receives chunk 0
+    assert torch.equal(b, torch.full((2,), 12.0))
+    assert mgr.cp_ring.deposited[(0, 0)] == {0, 1}
+    pgm.setup_process_group_manager(1, 1, 1, 1)
