@@ -9,8 +9,8 @@ chunks dense) and its backward adds into dK/dV of those chunks.  The four ranks 
 launch per direction: the grid's query-tile index enumerates (rank, tile of the rank's chunk), every
 workgroup walks the chunks its rank would receive, the online softmax carries across them (no score
 matrix, no per-chunk partial result and no separate merge pass touches HBM), and dK/dV of a chunk are
-summed over the ranks inside the kernel.  Launches per step: forward, delta pre-pass, backward,
-dq fp32 -> bf16.  The step is recorded once into a HIP graph and replayed K times; inputs are resident
+summed over the ranks inside the kernel.  Launches per step: forward, delta pre-pass, backward dK/dV,
+backward dQ (gradients are written in bf16 directly).  The step is recorded once into a HIP graph and replayed K times; inputs are resident
 in HBM before the timed region.
 
 value = algorithmic FLOPs of the step (7 * B*H*S^2*D = 60.13 GFLOP: forward 4 and backward 10 FLOPs
@@ -76,7 +76,7 @@ class RingBench:
         self.dv_acc = torch.empty(B, H, S, D, **f32)
         self.lse_b = torch.empty(B, H, S, **f32)
         self.delta_b = torch.empty(B, H, S, **f32)
-        self.dq_b = torch.empty(B, H, S, D, **f32)
+        self.dq_b = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=device)
         self.dk_b = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=device)
         self.dv_b = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=device)
 
@@ -101,7 +101,7 @@ class RingBench:
         for r in range(self.W):
             q, k, v, do, out, dk, dv = self._views(r)
             self.ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, self.dq_acc[r],
-                              dk, dv, accumulate=True)
+                              dk, dv, dkv_accumulate=True)
 
     def backward(self):
         self.dk_acc.zero_()
@@ -109,9 +109,9 @@ class RingBench:
         ops = self.ops
         for r in range(self.W):
             q, k, v, do, out, dk, dv = self._views(r)
-            delta = ops.attn_bwd_preprocess(do, out, self.dq_acc[r], delta=self.delta[r])
+            delta = ops.attn_bwd_preprocess(do, out, delta=self.delta[r])
             ops.attn_bwd(do, q, k, v, self.lse[r], delta, self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
-                         accumulate=True)
+                         dkv_accumulate=True)
         # hand the gradients back in the dtype of the inputs (autograd's cast in the reference)
         self.dq = [ops.convert_f32(self.dq_acc[r], self.torch.bfloat16) for r in range(self.W)]
         self.dk = ops.convert_f32(self.dk_acc, self.torch.bfloat16)
@@ -132,9 +132,8 @@ class RingBench:
     def step_batched(self):
         ops = self.ops
         self.forward_batched()
-        ops.attn_bwd_preprocess(self.do, self.out, self.dq_b, delta=self.delta_b)
+        ops.attn_bwd_preprocess(self.do, self.out, delta=self.delta_b)
         self.backward_kernel_batched()
-        self.dq_bf16 = ops.convert_f32(self.dq_b, self.torch.bfloat16)
 
     # -- the same work in the reference's shape: one launch per ring step (block + fused merge)
     def step_per_ring_step(self):
@@ -151,12 +150,12 @@ class RingBench:
                 ops.attn_fwd(q, self.k[:, :, c * Sc:(c + 1) * Sc], self.v[:, :, c * Sc:(c + 1) * Sc], self.scale, s == 0, 0,
                              out=out32, lse=lse, merge=s > 0)
             out = ops.convert_f32(out32, torch.bfloat16)
-            delta = ops.attn_bwd_preprocess(do, out, self.dq_acc[r])
+            delta = ops.attn_bwd_preprocess(do, out)
             for s in range(r + 1):
                 c = r - s
                 sl = slice(c * Sc, (c + 1) * Sc)
                 ops.attn_bwd(do, q, self.k[:, :, sl], self.v[:, :, sl], lse, delta, self.scale, s == 0, 0, self.dq_acc[r],
-                             self.dk_acc[:, :, sl], self.dv_acc[:, :, sl], accumulate=True)
+                             self.dk_acc[:, :, sl], self.dv_acc[:, :, sl], dq_accumulate=s > 0, dkv_accumulate=True)
         self.dq = [ops.convert_f32(self.dq_acc[r], torch.bfloat16) for r in range(self.W)]
         self.dk = ops.convert_f32(self.dk_acc, torch.bfloat16)
         self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
@@ -341,7 +340,7 @@ def main():
     # ---- dominant kernel: the backward launch alone, HIP events on the launching stream
     ms_bwd_k, _ = graph_time(torch, rb.backward_kernel_batched, max(args.steps // 2, 10))
     bwd_tflops = bwd_flops / (ms_bwd_k * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "attn_bwd_kernel_d64", "achieved": round(bwd_tflops, 2),
+    roofline = {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel_d64 + attn_bwd_dq_kernel (the two launches of pico_attn_bwd)", "achieved": round(bwd_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(bwd_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
                 "avg_launch_us": round(ms_bwd_k * 1e3, 2), "flops_per_launch": bwd_flops, "traffic": None}
 

@@ -146,25 +146,28 @@ int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, cons
 
 /* replaces: D = sum(dO * O, dim=-1)  context_parallel.py:145.
  * delta: [B,Hq,Sq] fp32.  out is addressed by o_stride like dout and has dtype out_dtype.
- * If dq_acc is not NULL the [B,Hq,Sq,D] contiguous fp32 buffer is zeroed in the same pass.
+ * If dq_acc is not NULL that [B,Hq,Sq,D] contiguous fp32 buffer is zeroed in the same pass (optional).
  */
 int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* dout, const void* out, int out_dtype,
                              float* delta, float* dq_acc, void* stream);
 
 /* replaces: ring_attention_backward  context_parallel.py:130-155 and the fp32 accumulation of
  *           RingAttentionFunc.backward  context_parallel.py:85-93.
+ * Two kernels are enqueued: dK/dV (one workgroup per 128 keys) and dQ (one workgroup per query tile);
+ * neither uses atomics, so results are deterministic.
  * lse, delta: [B,Hq,Sq] fp32 (lse is the FINAL merged lse, as in the reference).
- * dq_acc: [B,Hq,Sq,D] contiguous fp32, accumulated with atomic adds (zero it first, or keep the
- *         running sum across ring steps).
- * dk, dv: [B,Hkv,Sk,D] addressed by dkv_stride (element strides for b, h, s; NULL = contiguous);
- *         dkv_dtype PICO_F32 with accumulate = 1 adds into the buffers (the travelling fp32 accumulators
- *         of the ring), accumulate = 0 overwrites; PICO_BF16 overwrites.
- *         With Hq > Hkv the group's query heads are reduced inside the kernel.
+ * dq:     [B,Hq,Sq,D] addressed by dq_stride (element strides for b, h, s, multiples of 4; NULL = contiguous);
+ *         dq_dtype PICO_F32 with dq_accumulate = 1 adds into the buffer (the running sum over ring steps),
+ *         dq_accumulate = 0 overwrites; PICO_BF16 overwrites.
+ * dk, dv: [B,Hkv,Sk,D] addressed by dkv_stride (NULL = contiguous); same dtype / accumulate rules (the
+ *         travelling fp32 accumulators of the ring).  With Hq > Hkv the group's query heads are reduced
+ *         inside the kernel.
  */
 int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
                   const void* dout, const float* lse, const float* delta,
-                  float* dq_acc, void* dk, void* dv, const int64_t* dkv_stride,
-                  int dkv_dtype, int accumulate, void* stream);
+                  void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate,
+                  void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
+                  void* stream);
 
 /* fp32 -> bf16/fp32 conversion with layout change: src [B,H,S,D] contiguous fp32,
  * dst addressed by dst_stride (b,h,s).  Used to hand dq_acc back in the dtype / layout of q.

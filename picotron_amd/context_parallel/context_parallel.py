@@ -85,12 +85,12 @@ class RingAttentionFunc(torch.autograd.Function):
         world, rank, slot = ctx.cp_world, ctx.cp_rank, ctx.slot
         B, H, Sq, D = q.shape
 
-        dq = torch.empty(B, H, Sq, D, dtype=torch.float32, device=q.device)
-        delta = ops.attn_bwd_preprocess(dout, out, dq)  # also zeroes dq
+        delta = ops.attn_bwd_preprocess(dout, out)
 
         if world == 1:
-            dk, dv = ops.attn_bwd(dout, q, k, v, softmax_lse, delta, sm_scale, is_causal, 0, dq, dkv_dtype=k.dtype)
-            return ops.convert_f32(dq, q.dtype, like=q), dk, dv, None, None
+            dq, dk, dv = ops.attn_bwd(dout, q, k, v, softmax_lse, delta, sm_scale, is_causal, 0, dq_dtype=q.dtype,
+                                      dq_like=q, dkv_dtype=k.dtype)
+            return dq, dk, dv, None, None
 
         if not is_causal:
             raise NotImplementedError(
@@ -98,7 +98,7 @@ class RingAttentionFunc(torch.autograd.Function):
                 "one-rank-at-a-time replay cannot deliver; use ring_attention_backward per block instead")
         kv_comm = ContextCommunicate("kv_comm", rank=rank, slot=slot)
         d_kv_comm = ContextCommunicate("d_kv_comm", rank=rank, slot=slot)
-        dk = dv = None
+        dq = dk = dv = None
         next_dk = next_dv = None
         next_k = next_v = None
         for step in range(world):
@@ -110,14 +110,13 @@ class RingAttentionFunc(torch.autograd.Function):
                 bwd_causal = is_causal and step == 0
                 if dk is None:
                     # first block: fresh fp32 accumulators (:85-88)
-                    dk, dv = ops.attn_bwd(dout, q, k, v, softmax_lse, delta, sm_scale, bwd_causal, 0, dq,
-                                          dkv_dtype=torch.float32)
+                    dq, dk, dv = ops.attn_bwd(dout, q, k, v, softmax_lse, delta, sm_scale, bwd_causal, 0)
                 else:
-                    # dq += block_dq ; dk = block_dk + next_dk (:90-93), the adds happen inside the kernel
+                    # dq += block_dq ; dk = block_dk + next_dk (:90-93), the adds happen inside the kernels
                     d_kv_comm.wait()
                     dk, dv = next_dk, next_dv
                     ops.attn_bwd(dout, q, k, v, softmax_lse, delta, sm_scale, bwd_causal, 0, dq, dk, dv,
-                                 accumulate=True)
+                                 dq_accumulate=True, dkv_accumulate=True)
             elif step != 0:
                 d_kv_comm.wait()
                 dk, dv = next_dk, next_dv
@@ -145,12 +144,9 @@ def ring_attention_forward(q, k, v, sm_scale, is_causal):
 
 def ring_attention_backward(dO, Q, K, V, O, softmax_lse, sm_scale, is_causal):
     """Gradients of one block given the final (merged) O and lse; returns fp32 (dQ, dK, dV)."""
-    B, H, Sq, D = Q.shape
-    dq = torch.empty(B, H, Sq, D, dtype=torch.float32, device=Q.device)
-    delta = ops.attn_bwd_preprocess(dO, O, dq)
+    delta = ops.attn_bwd_preprocess(dO, O)
     lse = softmax_lse if softmax_lse.dtype == torch.float32 else softmax_lse.float()
-    dk, dv = ops.attn_bwd(dO, Q, K, V, lse, delta, sm_scale, is_causal, 0, dq, dkv_dtype=torch.float32)
-    return dq, dk, dv
+    return ops.attn_bwd(dO, Q, K, V, lse, delta, sm_scale, is_causal, 0)
 
 
 def update_out_and_lse(

@@ -1,28 +1,23 @@
-// Attention backward for gfx950 (MFMA bf16): one workgroup owns 128 keys of one kv head, keeps
-// dK / dV for them in registers, and walks over the query tiles (and the query heads of a GQA
-// group) that can see those keys.
+// Attention backward for gfx950 (MFMA bf16), split into two kernels so that no gradient needs atomics:
 //
-// Per 64-query tile:
-//   S  = Q K^T, dP = dO V^T          (C tile: lane = key, registers = queries; K, V fragments live
-//                                     in registers for the whole kernel)
-//   P  = exp2(S*c - lse*log2e),  dS = P * (dP - delta)
-//   dV += P^T dO,  dK += dS^T Q      (P / dS feed the MFMA straight from registers as the A operand;
-//                                     dO and Q come from the row-major LDS tiles through transposing reads)
-//   dS^T -> LDS, barrier
-//   dQ  = dS K * scale               (each wave owns 32x32 blocks of the 64 x D tile over all 128 keys; K
-//                                     fragments stay in registers, dS comes back through transposing
-//                                     LDS reads) -> fp32 atomic adds
+//  dK/dV kernel: one workgroup owns 128 keys of one kv head (32 per wave), keeps their K / V fragments and
+//    the dK / dV accumulators in registers, and walks over the 64-query tiles (and the query heads of a
+//    GQA group) that can see those keys:
+//      S = Q K^T, dP = dO V^T   (C tile: lane = key, registers = queries)
+//      P = exp2(S*c - lse*log2e),  dS = P * (dP - delta)
+//      dV += P^T dO,  dK += dS^T Q   (P / dS feed the MFMA straight from registers as A operands; dO and Q
+//                                     come from the row-major LDS tiles through transposing reads)
+//  dQ kernel: one workgroup owns 32 queries per wave, keeps Q / dO fragments, lse and delta in registers and
+//    walks over the K/V tiles like the forward kernel, in the transposed orientation (lane = query):
+//      S^T = K Q^T, dP^T = V dO^T,  dS^T = P^T * (dP^T - delta)  (lse / delta are per-lane scalars)
+//      dQ^T += K^T dS^T            (dS^T goes from the C registers into the B operand; K^T is read from the
+//                                   row-major K tile through transposing LDS reads)
+//
+// Recomputing S and dP in the second kernel costs 2 of 7 MFMA products; a single-kernel version that
+// accumulated dQ with fp32 atomics was bound by the atomic rate of the memory system (measured).
 #include "attn_common.h"
 
 #include <type_traits>
-
-#if defined(PICO_BWD_TIMING)
-__device__ long long pico_dbg[64];
-#define PICO_T(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && it == 2) pico_dbg[i] = clock64(); } while (0)
-extern "C" int pico_debug_read(long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(pico_dbg), sizeof(long long) * 64); }
-#else
-#define PICO_T(i)
-#endif
 
 namespace pico {
 namespace {
@@ -32,40 +27,35 @@ struct BwdParams {
   const __bf16* dout;
   const float* lse;
   const float* delta;
-  float* dq_acc;
+  void* dq;
   void* dk;
   void* dv;
-  int dkv_f32;
-  int accumulate;
+  int dq_f32, dq_accumulate;
+  int dkv_f32, dkv_accumulate;
+  int64_t dqs[3];  // element strides (b, h, s) of dq
   int64_t dks[3];  // element strides (b, h, s) of dk and dv
 };
 
+// =====================================================================================  dK / dV
 template <int D>
-struct BwdCfg {
+struct KvCfg {
   static constexpr int NW = 4;
   static constexpr int kThreads = 64 * NW;
   static constexpr int BN = 32 * NW;  // keys per workgroup
-  static constexpr int BM = 64;       // queries per iteration
-  static constexpr int LDQ = D + 8;   // pitch of the Q, dO and K tiles
-  static constexpr int LDS_ = BM + 8; // pitch of the dS^T tile [BN][BM]
+  static constexpr int BM = 64;       // queries per trip
+  static constexpr int LDQ = D + 8;   // pitch of the Q and dO tiles
   static constexpr int kVecPerRow = D / 8;
   static constexpr int kQLoads = BM * kVecPerRow / kThreads;
-  static constexpr int kKLoads = BN * kVecPerRow / kThreads;
-  static constexpr size_t kLdsBytes =
-      (2 * BM * LDQ + BN * LDQ + 2 * BN * LDS_) * sizeof(__bf16) + 2 * BM * sizeof(float);
+  static constexpr int kBufElems = 2 * BM * LDQ;                       // Q + dO tile of one stage (bf16)
+  static constexpr size_t kBufBytes = kBufElems * sizeof(__bf16) + 2 * BM * sizeof(float);
+  static constexpr size_t kLdsBytes = 2 * kBufBytes;                   // double-buffered
 };
 
 template <int D>
-__device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
-  using C = BwdCfg<D>;
-  constexpr int BM = C::BM, BN = C::BN, LDQ = C::LDQ, LDS_ = C::LDS_;
+__device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
+  using C = KvCfg<D>;
+  constexpr int BM = C::BM, BN = C::BN, LDQ = C::LDQ;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  __bf16* sQ = reinterpret_cast<__bf16*>(smem_raw);
-  __bf16* sdO = sQ + BM * LDQ;
-  __bf16* sK = sdO + BM * LDQ;
-  __bf16* sdS = sK + BN * LDQ;
-  float* sL = reinterpret_cast<float*>(sdS + 2 * BN * LDS_);  // sdS is double-buffered
-  float* sDelta = sL + BM;
 
   const AttnParams& a = p.a;
   // grid = (Hkv * B, key tiles): the x index runs fastest in dispatch order, so all heads of key tile 0
@@ -97,32 +87,6 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
       vf[s] = __builtin_bit_cast(bf16x8, rv);
     }
   }
-  // ---- K tile -> LDS (row-major, rows past Sk are zero) for the dQ product
-#pragma unroll
-  for (int i = 0; i < C::kKLoads; ++i) {
-    const int idx = tid + i * C::kThreads;
-    const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-    u32x4 raw = {0, 0, 0, 0};
-    if (key0 + r < a.Sk) raw = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key0 + r) * a.ks[2] + cv * 8);
-    *reinterpret_cast<u32x4*>(&sK[r * LDQ + cv * 8]) = raw;
-  }
-
-  // ---- K as the B operand of dQ = dS K (B[k = key][n = d]) for the dQ blocks this wave owns: read
-  //      once through transposing LDS reads and kept in registers
-  constexpr int kDqBlocks = (BM / 32) * (D / 32);
-  constexpr int kDqPasses = kDqBlocks / C::NW;
-  static_assert(kDqBlocks % C::NW == 0, "dQ blocks must split evenly over the waves");
-  bf16x8 ktf[kDqPasses][BN / 16];
-  __syncthreads();
-#pragma unroll
-  for (int pass = 0; pass < kDqPasses; ++pass) {
-    const int db_w = (pass * C::NW + wave) % (D / 32);
-#pragma unroll
-    for (int ks = 0; ks < BN / 16; ++ks) {
-      const int krow = 16 * ks + 4 * h + (lane % 16) / 4;
-      ktf[pass][ks] = lds_read_tr_pair(&sK[krow * LDQ + 32 * db_w + 16 * ((lane / 16) % 2) + 4 * (lane % 4)], LDQ);
-    }
-  }
 
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
 #pragma unroll
@@ -130,7 +94,7 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) { dk_acc[db][i] = 0.f; dv_acc[db][i] = 0.f; }
 
-  // ---- iteration space: (query head of the group) x (query tiles that can see key0)
+  // ---- trip space: (query head of the group) x (query tiles that can see key0)
   const int n_qtiles = (a.Sq + BM - 1) / BM;
   int qt_start = 0;
   if (a.causal) {
@@ -140,9 +104,9 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
   const int tiles_per_head = n_qtiles > qt_start ? n_qtiles - qt_start : 0;
   const int n_iter = tiles_per_head * group;
 
-  // Global -> register prefetch of the next Q / dO tile (+ lse, delta).  Loads are unconditional (rows
-  // past Sq are clamped to the last row and zeroed when they are written to LDS) and nothing here uses a
-  // loaded value, so the loop never has to wait for memory inside the prefetch.
+  // Global -> register prefetch of a Q / dO tile (+ lse, delta).  Loads are unconditional (rows past Sq
+  // are clamped and zeroed on the way into LDS) and nothing here uses a loaded value, so the loop holds
+  // no wait for memory other than the one in front of the LDS fill, a whole trip after the loads.
   u32x4 qreg[C::kQLoads], doreg[C::kQLoads];
   float lreg = 0.f, dreg = 0.f;
   auto prefetch = [&](int it) {
@@ -166,95 +130,53 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
       dreg = p.delta[gi];
     }
   };
-
-  if (n_iter > 0) prefetch(0);
-
-  // Software pipeline over the (head, query tile) pairs.  Trip `it` stages tile `it` in LDS and runs its
-  // S phase, and first finishes tile `it - 1`: its dS^T sits in the other half of the double-buffered
-  // sdS, so the dQ product and its atomics are issued a whole trip before anything waits on memory
-  // again, and one barrier per tile disappears.  The prefetch loads are issued after those atomics, so
-  // the wait before the next LDS fill covers operations that have had a full trip to complete.
-  int prev_hq = 0, prev_q0 = 0;
-  for (int it = 0; it <= n_iter; ++it) {
-    const bool have_tile = it < n_iter;
-    const int hq = hkv * group + (have_tile ? it / tiles_per_head : 0);
-    const int q0 = (qt_start + (have_tile ? it % tiles_per_head : 0)) * BM;
-    PICO_T(0);
-    __syncthreads();  // S phase of tile it-1 is complete: sdS[(it-1)&1] is full, sQ / sdO are free
-    PICO_T(1);
-    if (have_tile) {
+  auto stage = [&](int it, int buf) {
+    const int q0 = (qt_start + it % tiles_per_head) * BM;
+    __bf16* sQ = reinterpret_cast<__bf16*>(smem_raw + buf * C::kBufBytes);
+    __bf16* sdO = sQ + BM * LDQ;
+    float* sL = reinterpret_cast<float*>(sdO + BM * LDQ);
+    float* sDelta = sL + BM;
 #pragma unroll
-      for (int i = 0; i < C::kQLoads; ++i) {
-        const int idx = tid + i * C::kThreads;
-        const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-        const bool live = q0 + r < a.Sq;
-        const u32x4 zero = {0, 0, 0, 0};
-        *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = live ? qreg[i] : zero;
-        *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = live ? doreg[i] : zero;
-      }
-      if (tid < BM) {
-        // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
-        const bool live = q0 + tid < a.Sq && lreg != -INFINITY;
-        sL[tid] = live ? lreg * kLog2e : INFINITY;
-        sDelta[tid] = live ? dreg : 0.f;
-      }
+    for (int i = 0; i < C::kQLoads; ++i) {
+      const int idx = tid + i * C::kThreads;
+      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+      const bool live = q0 + r < a.Sq;
+      const u32x4 zero = {0, 0, 0, 0};
+      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = live ? qreg[i] : zero;
+      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = live ? doreg[i] : zero;
     }
-    PICO_T(2);
-    __syncthreads();
-    PICO_T(3);
-
-    // ================= dQ of the previous tile: the 64 x D tile is cut into 32 x 32 blocks, NW per pass
-#if !defined(PICO_BWD_NO_DQ)
-    if (it > 0) {
-      const __bf16* sdS_prev = sdS + ((it - 1) & 1) * (BN * LDS_);
-#pragma unroll
-      for (int pass = 0; pass < kDqPasses; ++pass) {
-        const int blk = pass * C::NW + wave;         // block index: query half x d block
-        const int qb_w = blk / (D / 32), db_w = blk % (D / 32);
-        f32x16 dq;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) dq[i] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < BN / 16; ++ks) {
-          // A[m = query][k = key]: slots 4jj+t <- keys 16ks + 8jj + 4h + t, read transposed from dS^T[key][query]
-          const int krow = 16 * ks + 4 * h + (lane % 16) / 4;
-          const bf16x8 af = lds_read_tr_pair(&sdS_prev[krow * LDS_ + 32 * qb_w + 16 * ((lane / 16) % 2) + 4 * (lane % 4)], LDS_);
-          dq = mfma32(af, ktf[pass][ks], dq);
-        }
-        // rows past Sq add 0 to the last valid row instead of branching around the atomic
-        float* dqp = p.dq_acc + ((static_cast<int64_t>(b) * a.Hq + prev_hq) * a.Sq) * D + 32 * db_w + n;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const int qrow = prev_q0 + 32 * qb_w + 8 * (i / 4) + 4 * h + (i % 4);
-          const bool live = qrow < a.Sq;
-          const float val = live ? dq[i] * a.sm_scale : 0.f;
-          float* dst = dqp + static_cast<int64_t>(live ? qrow : a.Sq - 1) * D;
-#if defined(PICO_BWD_NO_ATOMIC)
-          *dst = val;
-#else
-          unsafeAtomicAdd(dst, val);
-#endif
-        }
-      }
+    if (tid < BM) {
+      // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
+      const bool live = q0 + tid < a.Sq && lreg != -INFINITY;
+      sL[tid] = live ? lreg * kLog2e : INFINITY;
+      sDelta[tid] = live ? dreg : 0.f;
     }
-#endif
-    PICO_T(4);
-    if (!have_tile) break;
-    if (it + 1 < n_iter) prefetch(it + 1);
-    PICO_T(5);
+  };
 
-    // ================= S phase: this wave's 32 keys against the tile's 64 queries
-    __bf16* sdS_cur = sdS + (it & 1) * (BN * LDS_);
-    const int kw0 = key0 + 32 * wave;
+  if (n_iter > 0) {
+    prefetch(0);
+    stage(0, 0);
+    if (n_iter > 1) prefetch(1);
+  }
+  __syncthreads();
+
+  const int kw0 = key0 + 32 * wave;
+  for (int it = 0; it < n_iter; ++it) {
+    // stage tile it+1 into the other buffer (its readers finished before the barrier that ended trip it-1)
+    if (it + 1 < n_iter) {
+      stage(it + 1, (it + 1) & 1);
+      if (it + 2 < n_iter) prefetch(it + 2);
+    }
+    const int q0 = (qt_start + it % tiles_per_head) * BM;
+    const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + (it & 1) * C::kBufBytes);
+    const __bf16* sdO = sQ + BM * LDQ;
+    const float* sL = reinterpret_cast<const float*>(sdO + BM * LDQ);
+    const float* sDelta = sL + BM;
+
 #pragma unroll
     for (int sb = 0; sb < BM / 32; ++sb) {
-      const int qs_pos = a.q_offset + q0 + 32 * sb;  // position of the sub-block's first query
-      __bf16* ds_dst = &sdS_cur[(32 * wave + n) * LDS_ + 32 * sb + 4 * h];
-      if (a.causal && kw0 > qs_pos + 31) {  // every (query, key) pair of this 32x32 block is masked
-#pragma unroll
-        for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x2*>(ds_dst + 8 * j) = u32x2{0, 0};
-        continue;
-      }
+      const int qs_pos = a.q_offset + q0 + 32 * sb;       // position of the sub-block's first query
+      if (a.causal && kw0 > qs_pos + 31) continue;        // every (query, key) pair of this block is masked
       f32x16 s_acc, dp_acc;
 #pragma unroll
       for (int i = 0; i < 16; ++i) { s_acc[i] = 0.f; dp_acc[i] = 0.f; }
@@ -289,12 +211,9 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
       else softmax_grad(std::false_type{});
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
+        // registers 8cc+4jj+t hold queries 32sb + 16cc + 8jj + 4h + t: fetch dO / Q rows in that order
         const bf16x8 pf = pack8(s_acc, 8 * cc);
         const bf16x8 dsf = pack8(dp_acc, 8 * cc);
-        // dS^T[key][query]: registers 8cc+4jj+t hold queries 32sb + 16cc + 8jj + 4h + t
-        const u32x4 raw = __builtin_bit_cast(u32x4, dsf);
-        *reinterpret_cast<u32x2*>(ds_dst + 16 * cc) = u32x2{raw[0], raw[1]};
-        *reinterpret_cast<u32x2*>(ds_dst + 16 * cc + 8) = u32x2{raw[2], raw[3]};
         const int qr = 32 * sb + 16 * cc + 4 * h + (lane % 16) / 4;
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
@@ -306,9 +225,7 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
         }
       }
     }
-    PICO_T(6);
-    prev_hq = hq;
-    prev_q0 = q0;
+    __syncthreads();  // all waves are done with buffer it&1 (refilled in trip it+1) and tile it+1 is visible
   }
 
   // ---- epilogue: dK (scaled) and dV rows of this wave's keys.  In accumulate mode all reads of a block
@@ -329,7 +246,7 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
       float ok[16], ov[16];
 #pragma unroll
       for (int i = 0; i < 16; ++i) { ok[i] = 0.f; ov[i] = 0.f; }
-      if (p.accumulate) {
+      if (p.dkv_accumulate) {
 #pragma unroll
         for (int i = 0; i < 16; ++i)
           if (live[i]) { ok[i] = pk[off[i]]; ov[i] = pv[off[i]]; }
@@ -353,14 +270,209 @@ __device__ __forceinline__ void attn_bwd_body(const BwdParams& p) {
 
 // D = 64 fits two workgroups per CU (<= 256 registers per lane), which lets one workgroup's MFMA
 // work overlap the other's softmax / LDS phases; D = 128 needs the full register file.
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_kernel_d64(const BwdParams p) {
-  attn_bwd_body<64>(p);
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_dkdv_kernel_d64(const BwdParams p) {
+  attn_bwd_dkdv_body<64>(p);
 }
-__global__ __launch_bounds__(256) void attn_bwd_kernel_d128(const BwdParams p) { attn_bwd_body<128>(p); }
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel_d128(const BwdParams p) { attn_bwd_dkdv_body<128>(p); }
 
-template <int D> struct BwdKernel;
-template <> struct BwdKernel<64> { static constexpr auto fn = &attn_bwd_kernel_d64; };
-template <> struct BwdKernel<128> { static constexpr auto fn = &attn_bwd_kernel_d128; };
+template <int D> struct KvKernel;
+template <> struct KvKernel<64> { static constexpr auto fn = &attn_bwd_dkdv_kernel_d64; };
+template <> struct KvKernel<128> { static constexpr auto fn = &attn_bwd_dkdv_kernel_d128; };
+
+// =====================================================================================  dQ
+template <int D, int NW, int KT>
+struct DqCfg {
+  static constexpr int kThreads = 64 * NW;
+  static constexpr int BM = 32 * NW;       // queries per workgroup (32 per wave)
+  static constexpr int BN = 64;            // keys per compute step
+  static constexpr int LDK = D + 8;        // pitch of the K and V tiles
+  static constexpr int kVecPerRow = D / 8;
+  static constexpr int kLoads = KT * kVecPerRow / kThreads;
+  static constexpr int kTileElems = 2 * KT * LDK;
+  static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);  // double-buffered
+  static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
+};
+
+template <int D, int NW, int KT>
+__global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p) {
+  using C = DqCfg<D, NW, KT>;
+  constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
+
+  const AttnParams& a = p.a;
+  const int n_qtiles = (a.Sq + BM - 1) / BM;
+  // same dispatch order as the forward kernel: every head's last (longest) query tile first
+  const int qtile = n_qtiles - 1 - static_cast<int>(blockIdx.y);
+  const int hq = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
+  const int hkv = hq / (a.Hq / a.Hkv);
+  const int q0 = qtile * BM;
+  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int n = lane % 32, h = lane / 32;
+  const float c = a.sm_scale * kLog2e;
+
+  const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
+  const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
+
+  // ---- per-lane query: Q and dO fragments (B operands), lse and delta
+  const int qrow = q0 + wave * 32 + n;
+  const bool qlive = qrow < a.Sq;
+  bf16x8 qf[D / 16], dof[D / 16];
+  float lse2 = INFINITY, delta = 0.f;
+  {
+    const int64_t rq = qlive ? qrow : 0;
+    const __bf16* qsrc = a.q + b * a.qs[0] + hq * a.qs[1] + rq * a.qs[2] + 8 * h;
+    const __bf16* dsrc = p.dout + b * a.os[0] + hq * a.os[1] + rq * a.os[2] + 8 * h;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s) {
+      u32x4 rq4 = {0, 0, 0, 0}, rd4 = {0, 0, 0, 0};
+      if (qlive) {
+        rq4 = *reinterpret_cast<const u32x4*>(qsrc + 16 * s);
+        rd4 = *reinterpret_cast<const u32x4*>(dsrc + 16 * s);
+      }
+      qf[s] = __builtin_bit_cast(bf16x8, rq4);
+      dof[s] = __builtin_bit_cast(bf16x8, rd4);
+    }
+    if (qlive) {
+      const int64_t gi = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + qrow;
+      const float l = p.lse[gi];
+      lse2 = (l == -INFINITY) ? INFINITY : l * kLog2e;  // a row that saw no key contributes nothing
+      delta = p.delta[gi];
+    }
+  }
+
+  f32x16 dq[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dq[db][i] = 0.f;
+
+  // ---- key range of this query tile
+  const int q_hi = (q0 + BM < a.Sq ? q0 + BM : a.Sq);
+  int kv_end = a.Sk;
+  if (a.causal) {
+    const int vis = a.q_offset + q_hi;
+    kv_end = vis < a.Sk ? vis : a.Sk;
+    if (kv_end < 0) kv_end = 0;
+  }
+  const int ntiles = (kv_end + KT - 1) / KT;
+
+  u32x4 kreg[C::kLoads], vreg[C::kLoads];
+  auto load_tile = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < C::kLoads; ++i) {
+      const int idx = tid + i * C::kThreads;
+      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+      const int key = (k0 + r < a.Sk) ? k0 + r : a.Sk - 1;
+      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + cv * 8);
+      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + cv * 8);
+    }
+  };
+  auto store_tile = [&](int k0, int buf) {
+    __bf16* sK = smem + buf * C::kTileElems;
+    __bf16* sV = sK + KT * LDK;
+#pragma unroll
+    for (int i = 0; i < C::kLoads; ++i) {
+      const int idx = tid + i * C::kThreads;
+      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+      const bool live = k0 + r < a.Sk;
+      const u32x4 zero = {0, 0, 0, 0};
+      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = live ? kreg[i] : zero;
+      *reinterpret_cast<u32x4*>(&sV[r * LDK + cv * 8]) = live ? vreg[i] : zero;
+    }
+  };
+
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(0, 0);
+    if (ntiles > 1) load_tile(KT);
+  }
+  __syncthreads();
+
+  const int blk_q_lo = a.q_offset + q0 + wave * 32;  // position of this wave's first query
+  const int qpos = a.q_offset + qrow;
+  for (int t = 0; t < ntiles; ++t) {
+    if (t + 1 < ntiles) {
+      store_tile((t + 1) * KT, (t + 1) & 1);
+      if (t + 2 < ntiles) load_tile((t + 2) * KT);
+    }
+    const __bf16* sK = smem + (t & 1) * C::kTileElems;
+    const __bf16* sV = sK + KT * LDK;
+#pragma unroll
+    for (int sub = 0; sub < KT / BN; ++sub) {
+      const int k0 = t * KT + sub * BN;
+      if (k0 >= kv_end) break;
+      if (a.causal && k0 > blk_q_lo + 31) continue;  // the wave's whole 32x64 block is in the future
+      const __bf16* sKs = sK + sub * BN * LDK;
+      const __bf16* sVs = sV + sub * BN * LDK;
+      f32x16 s_acc[BN / 32], dp_acc[BN / 32];
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = 0.f; dp_acc[mb][i] = 0.f; }
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+          const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
+          const bf16x8 va = *reinterpret_cast<const bf16x8*>(&sVs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
+          s_acc[mb] = mfma32(ka, qf[s], s_acc[mb]);
+          dp_acc[mb] = mfma32(va, dof[s], dp_acc[mb]);
+        }
+      }
+      // dS^T = P^T * (dP^T - delta); keys past the diagonal are masked only in tiles that straddle it
+      // (rows of K / V past Sk are zero, so those keys add nothing to dQ)
+      const bool need_mask = a.causal && (k0 + BN - 1 > blk_q_lo);
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          float pv = fast_exp2(s_acc[mb][i] * c - lse2);
+          if (need_mask) {
+            const int key = k0 + 32 * mb + 8 * (i / 4) + 4 * h + (i % 4);
+            if (key > qpos) pv = 0.f;
+          }
+          dp_acc[mb][i] = pv * (dp_acc[mb][i] - delta);
+        }
+      // ---- dQ^T[d][query] += K^T[d][key] dS^T[key][query]
+#pragma unroll
+      for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+        for (int cc = 0; cc < 2; ++cc) {
+          const bf16x8 dsf = pack8(dp_acc[mb], 8 * cc);
+          const int krow = 32 * mb + 16 * cc + 4 * h + (lane % 16) / 4;
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db) {
+            const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+            const bf16x8 ktf = lds_read_tr_pair(&sKs[krow * LDK + col], LDK);
+            dq[db] = mfma32(ktf, dsf, dq[db]);
+          }
+        }
+    }
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane = query, registers = 4 consecutive d per (db, j)
+  if (!qlive) return;
+  const int64_t off = b * p.dqs[0] + hq * p.dqs[1] + static_cast<int64_t>(qrow) * p.dqs[2];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = 32 * db + 8 * j + 4 * h;
+      if (p.dq_f32) {
+        float* dst = static_cast<float*>(p.dq) + off + d;
+        f32x4 v4 = {0.f, 0.f, 0.f, 0.f};
+        if (p.dq_accumulate) v4 = *reinterpret_cast<const f32x4*>(dst);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) v4[t] += dq[db][4 * j + t] * a.sm_scale;
+        *reinterpret_cast<f32x4*>(dst) = v4;
+      } else {
+        u32x2 v2;
+        v2[0] = pack_bf16x2(dq[db][4 * j] * a.sm_scale, dq[db][4 * j + 1] * a.sm_scale);
+        v2[1] = pack_bf16x2(dq[db][4 * j + 2] * a.sm_scale, dq[db][4 * j + 3] * a.sm_scale);
+        *reinterpret_cast<u32x2*>(static_cast<__bf16*>(p.dq) + off + d) = v2;
+      }
+    }
+}
 
 // delta[row] = sum_d dO * O, one 16-byte vector of each per lane, D/8 lanes per row.
 template <int D, typename TO>
@@ -405,18 +517,37 @@ __global__ __launch_bounds__(256) void attn_bwd_preprocess_kernel(const __bf16* 
   if (row < rows && v == 0) delta[row] = part;
 }
 
+template <typename K>
+int set_lds(K kernel, size_t bytes, const char* what) {
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                          static_cast<int>(bytes)) != hipSuccess)
+    return fail(PICO_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", what, bytes);
+  return PICO_OK;
+}
+
 template <int D>
-int launch_bwd(const BwdParams& p, hipStream_t s) {
-  using C = BwdCfg<D>;
+int launch_dkdv(const BwdParams& p, hipStream_t s) {
+  using C = KvCfg<D>;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(BwdKernel<D>::fn),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(C::kLdsBytes)) != hipSuccess)
-      return fail(PICO_ERR_LAUNCH, "pico_attn_bwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
+    if (int rc = set_lds(KvKernel<D>::fn, C::kLdsBytes, "pico_attn_bwd(dk/dv)")) return rc;
     attr_set = true;
   }
   const int n_ktiles = (p.a.Sk + C::BN - 1) / C::BN;
-  hipLaunchKernelGGL(BwdKernel<D>::fn, dim3(p.a.Hkv * p.a.B, n_ktiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  hipLaunchKernelGGL(KvKernel<D>::fn, dim3(p.a.Hkv * p.a.B, n_ktiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  return PICO_OK;
+}
+
+template <int D, int NW, int KT>
+int launch_dq(const BwdParams& p, hipStream_t s) {
+  using C = DqCfg<D, NW, KT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (int rc = set_lds(&attn_bwd_dq_kernel<D, NW, KT>, C::kLdsBytes, "pico_attn_bwd(dq)")) return rc;
+    attr_set = true;
+  }
+  const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
+  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, NW, KT>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
   return PICO_OK;
 }
 
@@ -450,35 +581,64 @@ extern "C" int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* 
 }
 
 extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
-                             const float* lse, const float* delta, float* dq_acc, void* dk, void* dv,
-                             const int64_t* dkv_stride, int dkv_dtype, int accumulate, void* stream) {
+                             const float* lse, const float* delta, void* dq, const int64_t* dq_stride, int dq_dtype,
+                             int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
+                             int dkv_accumulate, void* stream) {
   if (int rc = check_attn_desc("pico_attn_bwd", desc)) return rc;
-  if (dkv_dtype != PICO_BF16 && dkv_dtype != PICO_F32)
-    return fail(PICO_ERR_DTYPE, "pico_attn_bwd: dk/dv dtype code %d not supported", dkv_dtype);
-  if (accumulate && dkv_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "pico_attn_bwd: accumulate needs fp32 dk/dv");
-  if (desc->B == 0 || desc->Sk == 0) return PICO_OK;  // no keys: nothing to add to dq, no dk/dv rows
-  if (!k || !v || !dk || !dv || (desc->Sq > 0 && (!q || !dout || !lse || !delta || !dq_acc)))
-    return fail(PICO_ERR_NULL, "pico_attn_bwd: q, k, v, dout, lse, delta, dq_acc, dk and dv are required");
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout))
-    return fail(PICO_ERR_ALIGN, "pico_attn_bwd: q, k, v and dout must be 16-byte aligned");
+  if ((dkv_dtype != PICO_BF16 && dkv_dtype != PICO_F32) || (dq_dtype != PICO_BF16 && dq_dtype != PICO_F32))
+    return fail(PICO_ERR_DTYPE, "pico_attn_bwd: gradient dtype codes %d / %d not supported", dq_dtype, dkv_dtype);
+  if ((dkv_accumulate && dkv_dtype != PICO_F32) || (dq_accumulate && dq_dtype != PICO_F32))
+    return fail(PICO_ERR_DTYPE, "pico_attn_bwd: accumulate needs fp32 gradients");
+  if (desc->B == 0) return PICO_OK;
+  const bool have_q = desc->Sq > 0, have_k = desc->Sk > 0;
+  if ((have_k && (!k || !v || !dk || !dv)) || (have_q && (!q || !dout || !lse || !delta || !dq)))
+    return fail(PICO_ERR_NULL, "pico_attn_bwd: q, k, v, dout, lse, delta, dq, dk and dv are required");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq))
+    return fail(PICO_ERR_ALIGN, "pico_attn_bwd: q, k, v, dout and dq must be 16-byte aligned");
   BwdParams p;
   p.a = make_params(desc, q, k, v);
   p.dout = static_cast<const __bf16*>(dout);
-  p.lse = lse; p.delta = delta; p.dq_acc = dq_acc; p.dk = dk; p.dv = dv;
+  p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.dq_f32 = dq_dtype == PICO_F32;
+  p.dq_accumulate = dq_accumulate != 0;
   p.dkv_f32 = dkv_dtype == PICO_F32;
-  p.accumulate = accumulate != 0;
-  if (dkv_stride) {
-    for (int i = 0; i < 3; ++i) {
-      if (dkv_stride[i] < 0) return fail(PICO_ERR_STRIDE, "pico_attn_bwd: negative dk/dv stride");
-      p.dks[i] = dkv_stride[i];
+  p.dkv_accumulate = dkv_accumulate != 0;
+  auto strides = [&](const int64_t* given, int heads, int seq, int64_t (&out)[3], int align) -> bool {
+    if (given) {
+      for (int i = 0; i < 3; ++i) {
+        if (given[i] < 0 || given[i] % align != 0) return false;
+        out[i] = given[i];
+      }
+    } else {
+      out[2] = desc->D;
+      out[1] = static_cast<int64_t>(seq) * desc->D;
+      out[0] = out[1] * heads;
     }
-  } else {
-    p.dks[2] = desc->D;
-    p.dks[1] = static_cast<int64_t>(desc->Sk) * desc->D;
-    p.dks[0] = p.dks[1] * desc->Hkv;
-  }
+    return true;
+  };
+  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, 4) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 1))
+    return fail(PICO_ERR_STRIDE, "pico_attn_bwd: dq strides must be non-negative multiples of 4, dk/dv strides non-negative");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int rc = desc->D == 64 ? launch_bwd<64>(p, s) : launch_bwd<128>(p, s);
-  if (rc) return rc;
-  return check_launch("pico_attn_bwd");
+  int rc = PICO_OK;
+  if (have_k) {
+    // without queries the dK/dV kernel still runs: it writes (or adds) zeros
+    rc = desc->D == 64 ? launch_dkdv<64>(p, s) : launch_dkdv<128>(p, s);
+    if (rc) return rc;
+    if (int lrc = check_launch("pico_attn_bwd(dk/dv)")) return lrc;
+  }
+  if (have_q) {
+    // without keys the dQ kernel still runs: it writes (or adds) zeros
+    if (desc->D == 64) {
+      const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
+      auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
+      if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
+      else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
+      else rc = launch_dq<64, 2, 64>(p, s);
+    } else {
+      rc = launch_dq<128, 4, 64>(p, s);
+    }
+    if (rc) return rc;
+    if (int lrc = check_launch("pico_attn_bwd(dq)")) return lrc;
+  }
+  return PICO_OK;
 }

@@ -8,6 +8,14 @@
 // 16-byte loads, V with transposing LDS reads (the contraction index of P V is V's row).
 #include "attn_common.h"
 
+#if defined(PICO_FWD_TIMING)
+__device__ long long pico_fdbg[64];
+#define PICO_FT(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && t == 2 && sub == 0) pico_fdbg[i] = clock64(); } while (0)
+extern "C" int pico_fwd_debug_read(long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(pico_fdbg), sizeof(long long) * 64); }
+#else
+#define PICO_FT(i)
+#endif
+
 namespace pico {
 namespace {
 
@@ -19,24 +27,36 @@ struct FwdParams {
   int merge;
 };
 
-template <int D, int QB, int NW>
+template <int D, int QB, int NW, int KT>
 struct FwdCfg {
   static constexpr int kThreads = 64 * NW;
   static constexpr int BM = 32 * QB * NW;  // queries per workgroup
-  static constexpr int BN = 64;            // keys per LDS tile
+  static constexpr int BN = 64;            // keys per compute step
+  static constexpr int kKT = KT;           // keys per staged LDS tile (a multiple of BN), double-buffered
   static constexpr int LDK = D + 8;        // K tile pitch: 16-byte row reads hit distinct banks
-  static constexpr int LDV = D + 32;       // V tile pitch: 4 rows x 64 bytes of a transposed read do
+#ifndef PICO_FWD_LDVPAD
+#define PICO_FWD_LDVPAD 8
+#endif
+  static constexpr int LDV = D + PICO_FWD_LDVPAD;  // V tile pitch for the 4-row transposing reads
   static constexpr int kVecPerRow = D / 8;
-  static constexpr int kLoads = BN * kVecPerRow / kThreads;  // 16-byte loads per thread per tensor
-  static_assert(BN * kVecPerRow % kThreads == 0, "tile must split evenly over the threads");
+  static constexpr int kLoads = KT * kVecPerRow / kThreads;  // 16-byte loads per thread per tensor
+  static constexpr int kTileElems = KT * (LDK + LDV);
+  static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);
+  static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
-template <int D, int QB, int NW>
-__global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(const FwdParams p) {
-  using C = FwdCfg<D, QB, NW>;
+#ifndef PICO_FWD_KT8
+#define PICO_FWD_KT8 64
+#endif
+#ifndef PICO_FWD_ATTR
+#define PICO_FWD_ATTR
+#endif
+template <int D, int QB, int NW, int KT>
+__global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const FwdParams p) {
+  using C = FwdCfg<D, QB, NW, KT>;
   constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK, LDV = C::LDV;
-  __shared__ __attribute__((aligned(16))) __bf16 sK[BN * LDK];
-  __shared__ __attribute__((aligned(16))) __bf16 sV[BN * LDV];
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
 
   const AttnParams& a = p.a;
   const int n_qtiles = (a.Sq + BM - 1) / BM;
@@ -110,114 +130,137 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(const FwdParams p) {
     kv_end = vis < a.Sk ? vis : a.Sk;
     if (kv_end < 0) kv_end = 0;
   }
-  const int ntiles = (kv_end + BN - 1) / BN;
+  const int ntiles = (kv_end + KT - 1) / KT;
 
-  // ---- global -> register staging of one K/V tile
+  // ---- global -> register -> LDS staging of one K/V tile of KT keys.  Loads are unconditional (rows
+  //      past Sk are clamped and zeroed on the way into LDS) so the loop body holds no wait for memory
+  //      other than the one in front of the LDS fill, a whole tile after the loads were issued.
   u32x4 kreg[C::kLoads], vreg[C::kLoads];
   auto load_tile = [&](int k0) {
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const int key = k0 + r;
-      u32x4 zk = {0, 0, 0, 0}, zv = {0, 0, 0, 0};
-      if (key < a.Sk) {
-        zk = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + cv * 8);
-        zv = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + cv * 8);
-      }
-      kreg[i] = zk;
-      vreg[i] = zv;
+      const int key = (k0 + r < a.Sk) ? k0 + r : a.Sk - 1;
+      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + cv * 8);
+      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + cv * 8);
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&](int k0, int buf) {
+    __bf16* sK = smem + buf * C::kTileElems;
+    __bf16* sV = sK + KT * LDK;
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = kreg[i];
-      *reinterpret_cast<u32x4*>(&sV[r * LDV + cv * 8]) = vreg[i];
+      const bool live = k0 + r < a.Sk;
+      const u32x4 zero = {0, 0, 0, 0};
+      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = live ? kreg[i] : zero;
+      *reinterpret_cast<u32x4*>(&sV[r * LDV + cv * 8]) = live ? vreg[i] : zero;
     }
   };
 
-  if (ntiles > 0) load_tile(0);
+  if (ntiles > 0) {
+    load_tile(0);
+    store_tile(0, 0);
+    if (ntiles > 1) load_tile(KT);
+  }
+  __syncthreads();
 
   for (int t = 0; t < ntiles; ++t) {
-    const int k0 = t * BN;
-    __syncthreads();  // everyone is done reading the previous tile
-    store_tile();
-    __syncthreads();
-    if (t + 1 < ntiles) load_tile(k0 + BN);
+    // stage tile t+1 into the other buffer (its readers finished before the barrier that ended trip t-1)
+    if (t + 1 < ntiles) {
+      store_tile((t + 1) * KT, (t + 1) & 1);
+      if (t + 2 < ntiles) load_tile((t + 2) * KT);
+    }
+    const __bf16* sK = smem + (t & 1) * C::kTileElems;
+    const __bf16* sV = sK + KT * LDK;
 
 #pragma unroll
-    for (int qb = 0; qb < QB; ++qb) {
-      const int blk_q_lo = a.q_offset + q0 + (wave * QB + qb) * 32;  // position of the block's first query
-      if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
-      // ---- S^T[key][query] for 64 keys x 32 queries
-      f32x16 s_acc[BN / 32];
+    for (int sub = 0; sub < KT / BN; ++sub) {
+      const int k0 = t * KT + sub * BN;
+      if (k0 >= kv_end) break;
+      const __bf16* sKs = sK + sub * BN * LDK;
+      const __bf16* sVs = sV + sub * BN * LDV;
 #pragma unroll
-      for (int mb = 0; mb < BN / 32; ++mb) {
+      for (int qb = 0; qb < QB; ++qb) {
+        const int blk_q_lo = a.q_offset + q0 + (wave * QB + qb) * 32;  // position of the block's first query
+        if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
+        PICO_FT(0);
+        // ---- S^T[key][query] for 64 keys x 32 queries
+        f32x16 s_acc[BN / 32];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+        for (int mb = 0; mb < BN / 32; ++mb) {
 #pragma unroll
-        for (int s = 0; s < D / 16; ++s) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sK[(32 * mb + n) * LDK + 16 * s + 8 * h]);
-          s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
+          for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+#pragma unroll
+          for (int s = 0; s < D / 16; ++s) {
+            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
+            s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
+          }
         }
-      }
-      // ---- mask (only for tiles that straddle the diagonal or the end of K)
-      const bool need_mask = (a.causal && k0 + BN - 1 > blk_q_lo) || (k0 + BN > a.Sk);
-      if (need_mask) {
-        const int qpos = a.causal ? a.q_offset + qrow[qb] : 0x7fffffff;
+        PICO_FT(1);
+        // ---- mask (only for tiles that straddle the diagonal or the end of K)
+        const bool need_mask = (a.causal && k0 + BN - 1 > blk_q_lo) || (k0 + BN > a.Sk);
+        if (need_mask) {
+          const int qpos = a.causal ? a.q_offset + qrow[qb] : 0x7fffffff;
+#pragma unroll
+          for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+              const int key = k0 + 32 * mb + 8 * (i / 4) + 4 * h + (i % 4);
+              if (key > qpos || key >= a.Sk) s_acc[mb][i] = -INFINITY;
+            }
+        }
+        PICO_FT(2);
+        // ---- online softmax
+        float mx = s_acc[0][0];
+#pragma unroll
+        for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
+        mx = half_max(mx);
+        const float m_new = fmaxf(m_run[qb], mx * c);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = fast_exp2(m_run[qb] - m_use);
+        m_run[qb] = m_new;
+        float psum = 0.f;
 #pragma unroll
         for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-            const int key = k0 + 32 * mb + 8 * (i / 4) + 4 * h + (i % 4);
-            if (key > qpos || key >= a.Sk) s_acc[mb][i] = -INFINITY;
+            const float pv = fast_exp2(s_acc[mb][i] * c - m_use);
+            s_acc[mb][i] = pv;
+            psum += pv;
           }
-      }
-      // ---- online softmax
-      float mx = s_acc[0][0];
+        l_run[qb] = l_run[qb] * alpha + psum;
+        if (__any(alpha != 1.f)) {
 #pragma unroll
-      for (int mb = 0; mb < BN / 32; ++mb)
+          for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
-      mx = half_max(mx);
-      const float m_new = fmaxf(m_run[qb], mx * c);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = fast_exp2(m_run[qb] - m_use);
-      m_run[qb] = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int mb = 0; mb < BN / 32; ++mb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float pv = fast_exp2(s_acc[mb][i] * c - m_use);
-          s_acc[mb][i] = pv;
-          psum += pv;
+            for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
         }
-      l_run[qb] = l_run[qb] * alpha + psum;
-      if (__any(alpha != 1.f)) {
+        PICO_FT(3);
+        // ---- O^T[d][query] += V^T[d][key] P^T[key][query]
 #pragma unroll
-        for (int db = 0; db < D / 32; ++db)
+        for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
-      }
-      // ---- O^T[d][query] += V^T[d][key] P^T[key][query]
+          for (int cc = 0; cc < 2; ++cc) {
+            const bf16x8 pf = pack8(s_acc[mb], 8 * cc);
+            const int krow = 32 * mb + 16 * cc + 4 * h + (lane % 16) / 4;
 #pragma unroll
-      for (int mb = 0; mb < BN / 32; ++mb)
-#pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          const bf16x8 pf = pack8(s_acc[mb], 8 * cc);
-          const int krow = 32 * mb + 16 * cc + 4 * h + (lane % 16) / 4;
-#pragma unroll
-          for (int db = 0; db < D / 32; ++db) {
-            const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
-            const bf16x8 vf = lds_read_tr_pair(&sV[krow * LDV + col], LDV);
-            o[qb][db] = mfma32(vf, pf, o[qb][db]);
+            for (int db = 0; db < D / 32; ++db) {
+              const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+              const bf16x8 vf = lds_read_tr_pair(&sVs[krow * LDV + col], LDV);
+              o[qb][db] = mfma32(vf, pf, o[qb][db]);
+            }
           }
-        }
+        PICO_FT(4);
+      }
     }
+    { const int sub = 0; PICO_FT(5); }
+    __syncthreads();  // all waves are done with buffer t&1 (it is refilled in trip t+1) and tile t+1 is visible
+    { const int sub = 0; PICO_FT(6); }
   }
 
   // ---- epilogue
@@ -250,11 +293,19 @@ __global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(const FwdParams p) {
   }
 }
 
-template <int D, int QB, int NW>
-void launch(const FwdParams& p, hipStream_t s) {
-  using C = FwdCfg<D, QB, NW>;
+template <int D, int QB, int NW, int KT>
+int launch(const FwdParams& p, hipStream_t s) {
+  using C = FwdCfg<D, QB, NW, KT>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, QB, NW, KT>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(C::kLdsBytes)) != hipSuccess)
+      return fail(PICO_ERR_LAUNCH, "pico_attn_fwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
+    attr_set = true;
+  }
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
-  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), 0, s, p);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW, KT>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  return PICO_OK;
 }
 
 }  // namespace
@@ -315,14 +366,16 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
   hipStream_t s = static_cast<hipStream_t>(stream);
   // Tile choice for D = 64: more waves per workgroup share each staged K/V tile (fewer barriers and
   // global loads per MFMA), but the launch still has to fill 256 CUs, so small problems get small tiles.
+  int rc;
   if (desc->D == 64) {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
-    if (groups(256) >= 512) launch<64, 1, 8>(p, s);
-    else if (groups(128) >= 512) launch<64, 1, 4>(p, s);
-    else launch<64, 1, 2>(p, s);
+    if (groups(256) >= 512) rc = launch<64, 1, 8, PICO_FWD_KT8>(p, s);
+    else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
+    else rc = launch<64, 1, 2, 64>(p, s);
   } else {
-    launch<128, 1, 4>(p, s);
+    rc = launch<128, 1, 4, 64>(p, s);
   }
+  if (rc) return rc;
   return check_launch("pico_attn_fwd");
 }

@@ -82,8 +82,8 @@ class FlashAttnFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout):
         q, k, v, out, lse = ctx.saved_tensors
-        B, H, S, D = q.shape
-        dq_acc = torch.empty(B, H, S, D, dtype=torch.float32, device=q.device)
-        delta = ops.attn_bwd_preprocess(dout, out, dq_acc)
-        dk, dv = ops.attn_bwd(dout, q, k, v, lse, delta, ctx.sm_scale, ctx.causal, 0, dq_acc, dkv_dtype=k.dtype)
-        return ops.convert_f32(dq_acc, q.dtype, like=q), dk, dv, None, None
+        delta = ops.attn_bwd_preprocess(dout, out)
+        # gradients come back in the dtype and memory layout of their inputs: no accumulation buffer, no cast pass
+        dq, dk, dv = ops.attn_bwd(dout, q, k, v, lse, delta, ctx.sm_scale, ctx.causal, 0, dq_dtype=q.dtype, dq_like=q,
+                                  dkv_dtype=k.dtype)
+        return dq, dk, dv, None, None

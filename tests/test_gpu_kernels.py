@@ -268,9 +268,8 @@ def test_attn_bwd(ops, device, B, Hq, Hkv, Sq, Sk, D, causal, q_offset):
     scale = 1 / math.sqrt(D)
     qd, kd, vd, dod = (t.to(device) for t in (q, k, v, do))
     out, lse = ops.attn_fwd(qd, kd, vd, scale, causal, q_offset)
-    dq_acc = torch.empty(B, Hq, Sq, D, dtype=torch.float32, device=device)
-    delta = ops.attn_bwd_preprocess(dod, out, dq_acc)
-    dk, dv = ops.attn_bwd(dod, qd, kd, vd, lse, delta, scale, causal, q_offset, dq_acc)
+    delta = ops.attn_bwd_preprocess(dod, out)
+    dq_acc, dk, dv = ops.attn_bwd(dod, qd, kd, vd, lse, delta, scale, causal, q_offset)
     # oracle: autograd through the fp32 closed form on the same bf16-rounded inputs
     qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
     w_o, _ = OR.full_attention_closed_form(qf, expand_kv(kf, Hq), expand_kv(vf, Hq), scale, causal, q_offset)
@@ -294,17 +293,50 @@ def test_attn_bwd_block_with_final_lse_and_accumulate(ops, device):
                                      w_o, w_l, r, 0.125, True)
     out_d, lse_d = w_o.to(torch.bfloat16).to(device), w_l.to(device)
     dq_acc = torch.empty(B, H, Sc, D, dtype=torch.float32, device=device)
-    delta = ops.attn_bwd_preprocess(do.to(device), out_d, dq_acc)
+    delta = ops.attn_bwd_preprocess(do.to(device), out_d, dq_acc)    # also zeroes dq_acc
     for _, held, run, blk_causal in OR.schedule(W, r, True):
         if not run:
             continue
         dk = torch.ones(B, H, Sc, D, dtype=torch.float32, device=device)   # pre-existing travelling accumulators
         dv = torch.full((B, H, Sc, D), 2.0, dtype=torch.float32, device=device)
         ops.attn_bwd(do.to(device), q_r.to(device), ks[held].to(device), vs[held].to(device), lse_d, delta, 0.125,
-                     blk_causal, 0, dq_acc, dk, dv, accumulate=True)
+                     blk_causal, 0, dq_acc, dk, dv, dq_accumulate=True, dkv_accumulate=True)
         assert rel_l2(dk - 1.0, contrib[held][0]) <= 1e-2
         assert rel_l2(dv - 2.0, contrib[held][1]) <= 1e-2
     assert rel_l2(dq_acc, w_dq) <= 1e-2
+
+
+def test_attn_bwd_bf16_strided_outputs_and_determinism(ops, device):
+    """dq written as bf16 in q's [B,S,H,D] memory; two runs are bit-identical (no atomics in the backward)."""
+    B, H, S, D = 2, 4, 192, 64
+    q_bshd = rnd(B, S, H, D, seed=80).to(torch.bfloat16).to(device)
+    qd = q_bshd.transpose(1, 2)
+    _, k, v = attn_inputs(B, H, H, S, S, D, seed=81)
+    do = rnd(B, H, S, D, seed=84).to(torch.bfloat16).to(device)
+    kd, vd = k.to(device), v.to(device)
+    out, lse = ops.attn_fwd(qd, kd, vd, 0.125, True)
+    delta = ops.attn_bwd_preprocess(do, out)
+    a = ops.attn_bwd(do, qd, kd, vd, lse, delta, 0.125, True, 0, dq_dtype=torch.bfloat16, dq_like=qd, dkv_dtype=torch.bfloat16)
+    b = ops.attn_bwd(do, qd, kd, vd, lse, delta, 0.125, True, 0, dq_dtype=torch.bfloat16, dq_like=qd, dkv_dtype=torch.bfloat16)
+    assert a[0].stride() == qd.stride() and a[0].dtype == torch.bfloat16
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    f = ops.attn_bwd(do, qd, kd, vd, lse, delta, 0.125, True, 0)
+    for x, y in zip(a, f):
+        assert rel_l2(x, y) <= 5e-3
+
+
+def test_attn_empty_inputs(ops, device):
+    """No queries or no keys: nothing faults; gradients of the side that exists are zero."""
+    z = torch.zeros(1, 2, 0, 64, dtype=torch.bfloat16, device=device)
+    x = rnd(1, 2, 40, 64, seed=85).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(z, x, x, 0.125, False)
+    assert out.shape == (1, 2, 0, 64)
+    out, lse = ops.attn_fwd(x, z, z, 0.125, False)
+    assert out.abs().max().item() == 0.0 and torch.isinf(lse).all()
+    delta = ops.attn_bwd_preprocess(x, out)
+    dq, dk, dv = ops.attn_bwd(x, x, z, z, lse, delta, 0.125, False, 0)
+    assert dq.abs().max().item() == 0.0 and dk.shape == (1, 2, 0, 64)
 
 
 def test_convert_f32(ops, device):
