@@ -39,6 +39,9 @@ if ROOT not in sys.path:
 
 MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes of one dK/dV launch at the bench shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy
+# kernel of known size (see profiles/); None until measured
+TRAFFIC_BYTES_DKDV = None
 
 
 def parse():
@@ -128,6 +131,14 @@ class RingBench:
     def backward_kernel_batched(self):
         self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, self.dq_b,
                           self.dk_b, self.dv_b)
+
+    def backward_dkdv_only(self):
+        self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, None,
+                          self.dk_b, self.dv_b, want_dq=False)
+
+    def backward_dq_only(self):
+        self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, self.dq_b,
+                          want_dkv=False)
 
     def step_batched(self):
         ops = self.ops
@@ -337,15 +348,24 @@ def main():
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     value = total_flops / (ms_per_step * 1e-3) / 1e12
 
-    # ---- dominant kernel: the backward launch alone, HIP events on the launching stream
-    ms_bwd_k, _ = graph_time(torch, rb.backward_kernel_batched, max(args.steps // 2, 10))
-    bwd_tflops = bwd_flops / (ms_bwd_k * 1e-3) / 1e12
-    roofline = {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel_d64 + attn_bwd_dq_kernel (the two launches of pico_attn_bwd)", "achieved": round(bwd_tflops, 2),
-                "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(bwd_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
-                "avg_launch_us": round(ms_bwd_k * 1e3, 2), "flops_per_launch": bwd_flops, "traffic": None}
+    # ---- dominant kernel: the dK/dV launch alone, HIP events on the launching stream.  Its algorithmic work
+    #      is 4 of the backward's 5 matrix products (S, dP, dV, dK): 8 FLOPs per (query, key, d) triple.
+    dkdv_flops = bwd_flops * 0.8
+    ms_dkdv, _ = graph_time(torch, rb.backward_dkdv_only, max(args.steps // 2, 10))
+    dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
+    roofline = {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel_d64", "achieved": round(dkdv_tflops, 2),
+                "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
+                "avg_launch_us": round(ms_dkdv * 1e3, 2), "flops_per_launch": dkdv_flops, "traffic": TRAFFIC_BYTES_DKDV}
 
     extras = {}
     if not args.no_extras:
+        ms_dq, _ = graph_time(torch, rb.backward_dq_only, max(args.steps // 2, 10))
+        ms_bwd_k, _ = graph_time(torch, rb.backward_kernel_batched, max(args.steps // 2, 10))
+        extras["attn_bwd_dq_kernel"] = {"us_per_launch": round(ms_dq * 1e3, 2),
+                                        "TFLOP/s_algorithmic": round(bwd_flops * 0.2 / (ms_dq * 1e-3) / 1e12, 2),
+                                        "TFLOP/s_executed": round(bwd_flops * 0.6 / (ms_dq * 1e-3) / 1e12, 2),
+                                        "note": "recomputes S and dP: executes 3 products for 1 algorithmic"}
+        extras["attn_bwd_both_kernels"] = {"us": round(ms_bwd_k * 1e3, 2), "TFLOP/s_algorithmic": round(bwd_flops / (ms_bwd_k * 1e-3) / 1e12, 2)}
         ms_fwd, _ = graph_time(torch, rb.forward_batched, max(args.steps // 2, 10))
         extras["attn_fwd_kernel"] = {"TFLOP/s": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2), "us_per_launch": round(ms_fwd * 1e3, 2),
                                      "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}

@@ -162,6 +162,7 @@ int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* dout, const
  * dk, dv: [B,Hkv,Sk,D] addressed by dkv_stride (NULL = contiguous); same dtype / accumulate rules (the
  *         travelling fp32 accumulators of the ring).  With Hq > Hkv the group's query heads are reduced
  *         inside the kernel.
+ * A gradient that is not wanted is passed as NULL (dq, or dk and dv together) and its kernel is skipped.
  */
 int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
                   const void* dout, const float* lse, const float* delta,

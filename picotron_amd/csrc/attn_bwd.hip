@@ -421,15 +421,22 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
       // dS^T = P^T * (dP^T - delta); keys past the diagonal are masked only in tiles that straddle it
       // (rows of K / V past Sk are zero, so those keys add nothing to dQ)
       const bool need_mask = a.causal && (k0 + BN - 1 > blk_q_lo);
+      if (need_mask) {
+        // the asm statement keeps this a real (wave-uniform) branch instead of per-element selects
+        asm volatile("; masked tile" ::: "memory");
+#pragma unroll
+        for (int mb = 0; mb < BN / 32; ++mb)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) {
+            const int key = k0 + 32 * mb + 8 * (i / 4) + 4 * h + (i % 4);
+            if (key > qpos) s_acc[mb][i] = -INFINITY;   // exp2(-inf) = 0
+          }
+      }
 #pragma unroll
       for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          float pv = fast_exp2(s_acc[mb][i] * c - lse2);
-          if (need_mask) {
-            const int key = k0 + 32 * mb + 8 * (i / 4) + 4 * h + (i % 4);
-            if (key > qpos) pv = 0.f;
-          }
+          const float pv = fast_exp2(s_acc[mb][i] * c - lse2);
           dp_acc[mb][i] = pv * (dp_acc[mb][i] - delta);
         }
       // ---- dQ^T[d][query] += K^T[d][key] dS^T[key][query]
@@ -590,9 +597,13 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
   if ((dkv_accumulate && dkv_dtype != PICO_F32) || (dq_accumulate && dq_dtype != PICO_F32))
     return fail(PICO_ERR_DTYPE, "pico_attn_bwd: accumulate needs fp32 gradients");
   if (desc->B == 0) return PICO_OK;
-  const bool have_q = desc->Sq > 0, have_k = desc->Sk > 0;
-  if ((have_k && (!k || !v || !dk || !dv)) || (have_q && (!q || !dout || !lse || !delta || !dq)))
-    return fail(PICO_ERR_NULL, "pico_attn_bwd: q, k, v, dout, lse, delta, dq, dk and dv are required");
+  // a gradient that is not wanted is passed as NULL and its kernel is skipped
+  const bool want_dq = dq != nullptr, want_dkv = dk != nullptr || dv != nullptr;
+  if (want_dkv && (!dk || !dv)) return fail(PICO_ERR_NULL, "pico_attn_bwd: dk and dv must be given together");
+  const bool have_q = desc->Sq > 0 && want_dq, have_k = desc->Sk > 0 && want_dkv;
+  if (((have_q || have_k) && desc->Sq > 0 && (!q || !dout || !lse || !delta)) ||
+      ((have_q || have_k) && desc->Sk > 0 && (!k || !v)))
+    return fail(PICO_ERR_NULL, "pico_attn_bwd: q, k, v, dout, lse and delta are required");
   if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq))
     return fail(PICO_ERR_ALIGN, "pico_attn_bwd: q, k, v, dout and dq must be 16-byte aligned");
   BwdParams p;

@@ -195,14 +195,21 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
           for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
 #pragma unroll
           for (int s = 0; s < D / 16; ++s) {
+#if defined(PICO_ABL_NOQK)
+            s_acc[mb][s] += static_cast<float>(qf[qb][s][mb]);
+#else
             const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
             s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
+#endif
           }
         }
         PICO_FT(1);
         // ---- mask (only for tiles that straddle the diagonal or the end of K)
         const bool need_mask = (a.causal && k0 + BN - 1 > blk_q_lo) || (k0 + BN > a.Sk);
         if (need_mask) {
+          // the asm statement keeps this a real (wave-uniform) branch: without it the compiler turns the
+          // block into per-element selects that every tile pays for
+          asm volatile("; masked tile" ::: "memory");
           const int qpos = a.causal ? a.q_offset + qrow[qb] : 0x7fffffff;
 #pragma unroll
           for (int mb = 0; mb < BN / 32; ++mb)
@@ -229,7 +236,11 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
         for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
+#if defined(PICO_ABL_NOEXP)
+            const float pv = s_acc[mb][i] * c - m_use;
+#else
             const float pv = fast_exp2(s_acc[mb][i] * c - m_use);
+#endif
             s_acc[mb][i] = pv;
             psum += pv;
           }
@@ -251,15 +262,21 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
               const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+#if defined(PICO_ABL_NOPV)
+              o[qb][db][0] += static_cast<float>(pf[0]);
+#else
               const bf16x8 vf = lds_read_tr_pair(&sVs[krow * LDV + col], LDV);
               o[qb][db] = mfma32(vf, pf, o[qb][db]);
+#endif
             }
           }
         PICO_FT(4);
       }
     }
     { const int sub = 0; PICO_FT(5); }
+#if !defined(PICO_ABL_NOBAR)
     __syncthreads();  // all waves are done with buffer t&1 (it is refilled in trip t+1) and tile t+1 is visible
+#endif
     { const int sub = 0; PICO_FT(6); }
   }
 
@@ -370,8 +387,11 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
   if (desc->D == 64) {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
+#ifndef PICO_FWD_FORCE_NW4
     if (groups(256) >= 512) rc = launch<64, 1, 8, PICO_FWD_KT8>(p, s);
-    else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
+    else
+#endif
+    if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
     else rc = launch<64, 1, 2, 64>(p, s);
   } else {
     rc = launch<128, 1, 4, 64>(p, s);

@@ -244,39 +244,47 @@ def _like_strided(t: torch.Tensor, ref: torch.Tensor) -> torch.Tensor:
 def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset: int = 0,
              dq: Optional[torch.Tensor] = None, dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None,
              dq_accumulate: bool = False, dkv_accumulate: bool = False, dq_dtype=torch.float32,
-             dkv_dtype=torch.float32, dq_like: Optional[torch.Tensor] = None):
+             dkv_dtype=torch.float32, dq_like: Optional[torch.Tensor] = None, want_dq: bool = True,
+             want_dkv: bool = True):
     """Gradients of one attention block; returns (dq [B,Hq,Sq,D], dk, dv [B,Hkv,Sk,D]).
 
     Buffers that are passed in are written in place (fp32 ones can be accumulated into: the running dq of a
     rank and the travelling dk / dv of the ring); missing ones are allocated in the requested dtype, dq with
-    the strides of `dq_like` if given.
+    the strides of `dq_like` if given.  want_dq / want_dkv = False skips that gradient (and its kernel).
     """
     _dev(dout, q, k, v, lse, delta, dq, dk, dv)
     q, k, v, dout = _attn_in(q, "q"), _attn_in(k, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
     B, Hq, Sq, D = q.shape
     Hkv, Sk = k.size(1), k.size(2)
-    if dq is None:
+    if dq is None and want_dq:
         if dq_accumulate:
             raise RuntimeError("attn_bwd: dq_accumulate=True needs an existing dq")
         if dq_like is not None and _dense(dq_like) and dq_like.stride(-1) == 1 and dq_like.shape == q.shape:
             dq = torch.empty_strided(q.shape, dq_like.stride(), dtype=dq_dtype, device=q.device)
         else:
             dq = torch.empty(B, Hq, Sq, D, dtype=dq_dtype, device=q.device)
-    if dk is None or dv is None:
+    if (dk is None or dv is None) and want_dkv:
         if dkv_accumulate:
             raise RuntimeError("attn_bwd: dkv_accumulate=True needs existing dk / dv")
         dk = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
         dv = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
-    if dk.dtype != dv.dtype or dk.stride() != dv.stride() or dk.stride(-1) != 1 or dq.stride(-1) != 1:
-        raise RuntimeError("attn_bwd: dk and dv must share dtype and strides; dq, dk, dv need a unit D stride")
+    if not want_dq:
+        dq = None
+    if not want_dkv:
+        dk = dv = None
+    if dk is not None and (dk.dtype != dv.dtype or dk.stride() != dv.stride() or dk.stride(-1) != 1):
+        raise RuntimeError("attn_bwd: dk and dv must share dtype and strides, with a unit D stride")
+    if dq is not None and dq.stride(-1) != 1:
+        raise RuntimeError("attn_bwd: dq needs a unit D stride")
     if lse.dtype != torch.float32 or delta.dtype != torch.float32:
         raise RuntimeError("attn_bwd: lse and delta must be fp32")
     d = _desc(q, k, v, dout, sm_scale, causal, q_offset)
-    dqs = (ctypes.c_int64 * 3)(dq.stride(0), dq.stride(1), dq.stride(2))
-    dks = (ctypes.c_int64 * 3)(dk.stride(0), dk.stride(1), dk.stride(2))
+    dqs = (ctypes.c_int64 * 3)(*(dq.stride()[:3] if dq is not None else (0, 0, 0)))
+    dks = (ctypes.c_int64 * 3)(*(dk.stride()[:3] if dk is not None else (0, 0, 0)))
     check(_lib.lib().pico_attn_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(lse.contiguous()),
-                                   _ptr(delta.contiguous()), _ptr(dq), dqs, _dt(dq, "dq"), int(dq_accumulate),
-                                   _ptr(dk), _ptr(dv), dks, _dt(dk, "dk/dv"), int(dkv_accumulate), _stream()))
+                                   _ptr(delta.contiguous()), _ptr(dq), dqs, _dt(dq, "dq") if dq is not None else PICO_F32,
+                                   int(dq_accumulate), _ptr(dk), _ptr(dv), dks,
+                                   _dt(dk, "dk/dv") if dk is not None else PICO_F32, int(dkv_accumulate), _stream()))
     return dq, dk, dv
 
 
