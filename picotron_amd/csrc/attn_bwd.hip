@@ -409,7 +409,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
 #pragma unroll
       for (int mb = 0; mb < BN / 32; ++mb) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = 0.f; dp_acc[mb][i] = 0.f; }
+        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = 0.f; dp_acc[mb][i] = -delta; }  // dP - delta comes out of the MFMA
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) {
           const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
@@ -437,7 +437,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
           const float pv = fast_exp2(s_acc[mb][i] * c - lse2);
-          dp_acc[mb][i] = pv * (dp_acc[mb][i] - delta);
+          dp_acc[mb][i] = pv * dp_acc[mb][i];
         }
       // ---- dQ^T[d][query] += K^T[d][key] dS^T[key][query]
 #pragma unroll
@@ -646,7 +646,9 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
       else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
       else rc = launch_dq<64, 2, 64>(p, s);
     } else {
-      rc = launch_dq<128, 4, 64>(p, s);
+      const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
+      if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch_dq<128, 8, 64>(p, s);
+      else rc = launch_dq<128, 4, 64>(p, s);
     }
     if (rc) return rc;
     if (int lrc = check_launch("pico_attn_bwd(dq)")) return lrc;

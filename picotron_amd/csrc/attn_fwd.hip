@@ -8,14 +8,6 @@
 // 16-byte loads, V with transposing LDS reads (the contraction index of P V is V's row).
 #include "attn_common.h"
 
-#if defined(PICO_FWD_TIMING)
-__device__ long long pico_fdbg[64];
-#define PICO_FT(i) do { if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0 && t == 2 && sub == 0) pico_fdbg[i] = clock64(); } while (0)
-extern "C" int pico_fwd_debug_read(long long* out) { return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(pico_fdbg), sizeof(long long) * 64); }
-#else
-#define PICO_FT(i)
-#endif
-
 namespace pico {
 namespace {
 
@@ -186,7 +178,6 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
       for (int qb = 0; qb < QB; ++qb) {
         const int blk_q_lo = a.q_offset + q0 + (wave * QB + qb) * 32;  // position of the block's first query
         if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
-        PICO_FT(0);
         // ---- S^T[key][query] for 64 keys x 32 queries
         f32x16 s_acc[BN / 32];
 #pragma unroll
@@ -195,15 +186,10 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
           for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
 #pragma unroll
           for (int s = 0; s < D / 16; ++s) {
-#if defined(PICO_ABL_NOQK)
-            s_acc[mb][s] += static_cast<float>(qf[qb][s][mb]);
-#else
             const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
             s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
-#endif
           }
         }
-        PICO_FT(1);
         // ---- mask (only for tiles that straddle the diagonal or the end of K)
         const bool need_mask = (a.causal && k0 + BN - 1 > blk_q_lo) || (k0 + BN > a.Sk);
         if (need_mask) {
@@ -219,39 +205,37 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
               if (key > qpos || key >= a.Sk) s_acc[mb][i] = -INFINITY;
             }
         }
-        PICO_FT(2);
-        // ---- online softmax
+        // ---- online softmax.  The running maximum is only raised (and O, l rescaled) when some query of
+        //      the wave saw its maximum grow by more than 2^kTau; until then exp2(s - m) may exceed 1 by at
+        //      most that factor, which fp32 accumulators and bf16 probabilities hold without loss.
+        constexpr float kTau = 8.f;
         float mx = s_acc[0][0];
 #pragma unroll
         for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s_acc[mb][i]);
-        mx = half_max(mx);
-        const float m_new = fmaxf(m_run[qb], mx * c);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = fast_exp2(m_run[qb] - m_use);
-        m_run[qb] = m_new;
+        mx = half_max(mx) * c;
+        if (__any(mx > m_run[qb] + kTau)) {
+          const float m_new = fmaxf(m_run[qb], mx);
+          const float alpha = (m_new == -INFINITY) ? 1.f : fast_exp2(m_run[qb] - m_new);
+          m_run[qb] = m_new;
+#pragma unroll
+          for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
+          l_run[qb] *= alpha;
+        }
+        const float m_use = (m_run[qb] == -INFINITY) ? 0.f : m_run[qb];
         float psum = 0.f;
 #pragma unroll
         for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
           for (int i = 0; i < 16; ++i) {
-#if defined(PICO_ABL_NOEXP)
-            const float pv = s_acc[mb][i] * c - m_use;
-#else
             const float pv = fast_exp2(s_acc[mb][i] * c - m_use);
-#endif
             s_acc[mb][i] = pv;
             psum += pv;
           }
-        l_run[qb] = l_run[qb] * alpha + psum;
-        if (__any(alpha != 1.f)) {
-#pragma unroll
-          for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[qb][db][i] *= alpha;
-        }
-        PICO_FT(3);
+        l_run[qb] += psum;
         // ---- O^T[d][query] += V^T[d][key] P^T[key][query]
 #pragma unroll
         for (int mb = 0; mb < BN / 32; ++mb)
@@ -262,22 +246,13 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
 #pragma unroll
             for (int db = 0; db < D / 32; ++db) {
               const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
-#if defined(PICO_ABL_NOPV)
-              o[qb][db][0] += static_cast<float>(pf[0]);
-#else
               const bf16x8 vf = lds_read_tr_pair(&sVs[krow * LDV + col], LDV);
               o[qb][db] = mfma32(vf, pf, o[qb][db]);
-#endif
             }
           }
-        PICO_FT(4);
       }
     }
-    { const int sub = 0; PICO_FT(5); }
-#if !defined(PICO_ABL_NOBAR)
     __syncthreads();  // all waves are done with buffer t&1 (it is refilled in trip t+1) and tile t+1 is visible
-#endif
-    { const int sub = 0; PICO_FT(6); }
   }
 
   // ---- epilogue
@@ -387,14 +362,13 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
   if (desc->D == 64) {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
-#ifndef PICO_FWD_FORCE_NW4
     if (groups(256) >= 512) rc = launch<64, 1, 8, PICO_FWD_KT8>(p, s);
-    else
-#endif
-    if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
+    else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
     else rc = launch<64, 1, 2, 64>(p, s);
   } else {
-    rc = launch<128, 1, 4, 64>(p, s);
+    const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
+    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<128, 1, 8, 64>(p, s);
+    else rc = launch<128, 1, 4, 64>(p, s);
   }
   if (rc) return rc;
   return check_launch("pico_attn_fwd");
