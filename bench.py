@@ -41,7 +41,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one dK/dV launch at the bench shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy
 # kernel of known size (see profiles/); None until measured
-TRAFFIC_BYTES_DKDV = None
+TRAFFIC_BYTES_DKDV = 123.3e6
 
 
 def parse():
@@ -52,6 +52,9 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels")
     ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B-shaped training step")
+    ap.add_argument("--probe", action="store_true",
+                    help="counter probe: a few launches of a plain copy of known size and of each attention kernel "
+                         "at the bench shape, nothing else (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -322,6 +325,20 @@ def main():
     ops._lib.lib()  # fail loudly now if the HIP library is not built
 
     rb = RingBench(torch, ops)
+    if args.probe:
+        # plain copy of 64 MiB fp32 (read 64 MiB, write 64 MiB) as the scale for the HBM counters
+        src = torch.randn(16, 1024, 1024, dtype=torch.float32, device="cuda").view(1, 16, 1024, 1024)
+        for _ in range(5):
+            ops.convert_f32(src, torch.float32)
+        rb.forward_batched()
+        ops.attn_bwd_preprocess(rb.do, rb.out, delta=rb.delta_b)
+        for _ in range(5):
+            rb.forward_batched()
+            rb.backward_dkdv_only()
+            rb.backward_dq_only()
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "convert_kernel<float> copies 67108864 B in and out per launch; attention kernels at configs[1]"}))
+        return
     fwd_flops, bwd_flops = rb.flops()
     total_flops = fwd_flops + bwd_flops
 
