@@ -293,6 +293,51 @@ def train_step_extra(torch, steps=8, warmup=3):
     return res
 
 
+def long_context_extra(torch, ops, iters=10):
+    """configs[4]: rank 7 of cp 8 at total seq 32768 -- 4096 queries over 8 K/V chunks of 4096, GQA 32/8, head_dim 128,
+    forward + backward; 7.5 chunk-blocks of 14 * Hq * Sc^2 * D FLOP each = 7.215 TFLOP."""
+    W, Sc, Hq, Hkv, D, r = 8, 4096, 32, 8, 128, 7
+    scale = 1.0 / math.sqrt(D)
+    g = torch.Generator().manual_seed(0)
+    q = (torch.randn(1, Hq, Sc, D, generator=g) * scale).to(torch.bfloat16).cuda()
+    k, v = (torch.randn(1, Hkv, W * Sc, D, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+    do = torch.randn(1, Hq, Sc, D, generator=g).to(torch.bfloat16).cuda()
+    out = torch.empty_like(q)
+    lse = torch.empty(1, Hq, Sc, dtype=torch.float32, device="cuda")
+    delta = torch.empty_like(lse)
+    dq = torch.empty_like(q)
+    dk, dv = torch.empty_like(k), torch.empty_like(v)
+    flops = 7.5 * 14 * Hq * Sc * Sc * D
+
+    def fused():
+        ops.attn_fwd(q, k, v, scale, True, r * Sc, out=out, lse=lse)
+        ops.attn_bwd_preprocess(do, out, delta=delta)
+        ops.attn_bwd(do, q, k, v, lse, delta, scale, True, r * Sc, dq, dk, dv)
+
+    o32 = torch.empty(1, Hq, Sc, D, dtype=torch.float32, device="cuda")
+    dq32 = torch.empty_like(o32)
+    dk32 = torch.empty(1, Hkv, W * Sc, D, dtype=torch.float32, device="cuda")
+    dv32 = torch.empty_like(dk32)
+
+    def per_ring_step():
+        dk32.zero_()
+        dv32.zero_()
+        for s_ in range(W):
+            cs = slice((r - s_) * Sc, (r - s_ + 1) * Sc)
+            ops.attn_fwd(q, k[:, :, cs], v[:, :, cs], scale, s_ == 0, 0, out=o32, lse=lse, merge=s_ > 0)
+        ob = ops.convert_f32(o32, torch.bfloat16)
+        ops.attn_bwd_preprocess(do, ob, delta=delta)
+        for s_ in range(W):
+            cs = slice((r - s_) * Sc, (r - s_ + 1) * Sc)
+            ops.attn_bwd(do, q, k[:, :, cs], v[:, :, cs], lse, delta, scale, s_ == 0, 0, dq32, dk32[:, :, cs], dv32[:, :, cs],
+                         dq_accumulate=s_ > 0, dkv_accumulate=True)
+
+    ms_f, _ = graph_time(torch, fused, iters)
+    ms_r, _ = graph_time(torch, per_ring_step, iters)
+    return {"flops": flops, "one_launch_per_direction": {"ms": round(ms_f, 3), "TFLOP/s": round(flops / (ms_f * 1e-3) / 1e12, 1)},
+            "one_launch_per_ring_step": {"ms": round(ms_r, 3), "TFLOP/s": round(flops / (ms_r * 1e-3) / 1e12, 1)}}
+
+
 def cpu_baseline(host_tensors, W, scale, flops_total):
     """The CPU oracle on the same inputs: full configs[1] shape, fp32, all host threads and one thread."""
     import torch
@@ -396,6 +441,7 @@ def main():
         torch.cuda.synchronize()
         extras["eager_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / 20, 4)
         extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
+        extras["configs4_long_context_rank7_of_8"] = long_context_extra(torch, ops)
         if not args.no_train:
             extras["smollm_1p7b_train_step"] = train_step_extra(torch)
 
