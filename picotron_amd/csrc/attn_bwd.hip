@@ -104,30 +104,47 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
   const int tiles_per_head = n_qtiles > qt_start ? n_qtiles - qt_start : 0;
   const int n_iter = tiles_per_head * group;
 
-  // Global -> register prefetch of a Q / dO tile (+ lse, delta).  Loads are unconditional (rows past Sq
-  // are clamped and zeroed on the way into LDS) and nothing here uses a loaded value, so the loop holds
-  // no wait for memory other than the one in front of the LDS fill, a whole trip after the loads.
+  // Global -> register prefetch of a Q / dO tile (+ lse, delta).  Nothing here uses a loaded value, so the
+  // loop holds no wait for memory other than the one in front of the LDS fill, a whole trip after the
+  // loads.  Addresses are a wave-uniform base (head, first row of the tile) plus a per-thread byte offset
+  // that is computed once; only a tile that sticks out past Sq takes the path with clamped rows.
   u32x4 qreg[C::kQLoads], doreg[C::kQLoads];
   float lreg = 0.f, dreg = 0.f;
+  uint32_t q_off[C::kQLoads], do_off[C::kQLoads];
+#pragma unroll
+  for (int i = 0; i < C::kQLoads; ++i) {
+    const int idx = tid + i * C::kThreads;
+    const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+    q_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.qs[2] + cv * 8) * 2);
+    do_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.os[2] + cv * 8) * 2);
+  }
   auto prefetch = [&](int it) {
     const int hq = hkv * group + it / tiles_per_head;
     const int q0 = (qt_start + it % tiles_per_head) * BM;
-    const __bf16* qb = a.q + b * a.qs[0] + hq * a.qs[1];
-    const __bf16* dob = p.dout + b * a.os[0] + hq * a.os[1];
+    const char* qb = reinterpret_cast<const char*>(a.q + b * a.qs[0] + hq * a.qs[1] + static_cast<int64_t>(q0) * a.qs[2]);
+    const char* dob = reinterpret_cast<const char*>(p.dout + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(q0) * a.os[2]);
+    const int64_t row0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + q0;
+    if (q0 + BM <= a.Sq) {
 #pragma unroll
-    for (int i = 0; i < C::kQLoads; ++i) {
-      const int idx = tid + i * C::kThreads;
-      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const int row = (q0 + r < a.Sq) ? q0 + r : a.Sq - 1;
-      qreg[i] = *reinterpret_cast<const u32x4*>(qb + static_cast<int64_t>(row) * a.qs[2] + cv * 8);
-      doreg[i] = *reinterpret_cast<const u32x4*>(dob + static_cast<int64_t>(row) * a.os[2] + cv * 8);
-    }
-    {
-      const int r = tid % BM;
-      const int row = (q0 + r < a.Sq) ? q0 + r : a.Sq - 1;
-      const int64_t gi = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + row;
-      lreg = p.lse[gi];
-      dreg = p.delta[gi];
+      for (int i = 0; i < C::kQLoads; ++i) {
+        qreg[i] = *reinterpret_cast<const u32x4*>(qb + q_off[i]);
+        doreg[i] = *reinterpret_cast<const u32x4*>(dob + do_off[i]);
+      }
+      lreg = p.lse[row0 + tid % BM];
+      dreg = p.delta[row0 + tid % BM];
+    } else {
+      const int last = a.Sq - 1 - q0;  // last live row of the tile
+#pragma unroll
+      for (int i = 0; i < C::kQLoads; ++i) {
+        const int idx = tid + i * C::kThreads;
+        const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+        const int rc = r < last ? r : last;
+        qreg[i] = *reinterpret_cast<const u32x4*>(qb + (static_cast<int64_t>(rc) * a.qs[2] + cv * 8) * 2);
+        doreg[i] = *reinterpret_cast<const u32x4*>(dob + (static_cast<int64_t>(rc) * a.os[2] + cv * 8) * 2);
+      }
+      const int rl = (tid % BM) < last ? (tid % BM) : last;
+      lreg = p.lse[row0 + rl];
+      dreg = p.delta[row0 + rl];
     }
   };
   auto stage = [&](int it, int buf) {
@@ -136,20 +153,21 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     __bf16* sdO = sQ + BM * LDQ;
     float* sL = reinterpret_cast<float*>(sdO + BM * LDQ);
     float* sDelta = sL + BM;
+    const bool full = q0 + BM <= a.Sq;
 #pragma unroll
     for (int i = 0; i < C::kQLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const bool live = q0 + r < a.Sq;
-      const u32x4 zero = {0, 0, 0, 0};
-      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = live ? qreg[i] : zero;
-      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = live ? doreg[i] : zero;
+      u32x4 qv = qreg[i], dv4 = doreg[i];
+      if (!full && q0 + r >= a.Sq) { qv = u32x4{0, 0, 0, 0}; dv4 = u32x4{0, 0, 0, 0}; }
+      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = qv;
+      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = dv4;
     }
     if (tid < BM) {
       // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
       const bool live = q0 + tid < a.Sq && lreg != -INFINITY;
       sL[tid] = live ? lreg * kLog2e : INFINITY;
-      sDelta[tid] = live ? dreg : 0.f;
+      sDelta[tid] = live ? -dreg : 0.f;   // stored negated: it is loaded straight into the dP accumulator
     }
   };
 
@@ -177,9 +195,15 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     for (int sb = 0; sb < BM / 32; ++sb) {
       const int qs_pos = a.q_offset + q0 + 32 * sb;       // position of the sub-block's first query
       if (a.causal && kw0 > qs_pos + 31) continue;        // every (query, key) pair of this block is masked
+      // the dP accumulator starts at -delta of its row (sDelta holds the negated value), so dP - delta
+      // comes out of the MFMA
       f32x16 s_acc, dp_acc;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { s_acc[i] = 0.f; dp_acc[i] = 0.f; }
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) { s_acc[4 * j + t] = 0.f; dp_acc[4 * j + t] = d4[t]; }
+      }
 #pragma unroll
       for (int s = 0; s < D / 16; ++s) {
         const bf16x8 qa = *reinterpret_cast<const bf16x8*>(&sQ[(32 * sb + n) * LDQ + 16 * s + 8 * h]);
@@ -187,14 +211,14 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
         s_acc = mfma32(qa, kf[s], s_acc);
         dp_acc = mfma32(da, vf[s], dp_acc);
       }
-      // P = exp2(S*c - lse*log2e), dS = P * (dP - delta); the mask test is paid only on the diagonal
+      // P = exp2(S*c - lse*log2e), dS = P * (dP - delta) [already in the accumulator]; the mask test is paid
+      // only on the diagonal
       auto softmax_grad = [&](auto mask_c) {
         constexpr bool kMask = decltype(mask_c)::value;
         const int key_rel = kw0 + n - qs_pos - 4 * h;  // key is masked for row (8j + 4h + t) iff key_rel > 8j + t
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
-          const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
           for (int t = 0; t < 4; ++t) {
             const int i = 4 * j + t;
@@ -203,7 +227,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
               if (key_rel > 8 * j + t) pv = 0.f;
             }
             s_acc[i] = pv;
-            dp_acc[i] = pv * (dp_acc[i] - d4[t]);
+            dp_acc[i] = pv * dp_acc[i];
           }
         }
       };
