@@ -104,10 +104,10 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
   const int tiles_per_head = n_qtiles > qt_start ? n_qtiles - qt_start : 0;
   const int n_iter = tiles_per_head * group;
 
-  // Global -> register prefetch of a Q / dO tile (+ lse, delta).  Nothing here uses a loaded value, so the
-  // loop holds no wait for memory other than the one in front of the LDS fill, a whole trip after the
-  // loads.  Addresses are a wave-uniform base (head, first row of the tile) plus a per-thread byte offset
-  // that is computed once; only a tile that sticks out past Sq takes the path with clamped rows.
+  // Global -> register prefetch of a Q / dO tile (+ lse, delta) with buffer loads: the resource is rebuilt
+  // per tile from wave-uniform values (head, first row, rows left in the sequence), the per-lane byte
+  // offsets are computed once, and rows past Sq read as zeros.  Nothing here uses a loaded value, so the
+  // loop holds no wait for memory other than the one in front of the LDS fill, a whole trip after the loads.
   u32x4 qreg[C::kQLoads], doreg[C::kQLoads];
   float lreg = 0.f, dreg = 0.f;
   uint32_t q_off[C::kQLoads], do_off[C::kQLoads];
@@ -118,34 +118,25 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     q_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.qs[2] + cv * 8) * 2);
     do_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.os[2] + cv * 8) * 2);
   }
+  const uint32_t row_off = static_cast<uint32_t>((tid % BM) * 4);
   auto prefetch = [&](int it) {
     const int hq = hkv * group + it / tiles_per_head;
     const int q0 = (qt_start + it % tiles_per_head) * BM;
-    const char* qb = reinterpret_cast<const char*>(a.q + b * a.qs[0] + hq * a.qs[1] + static_cast<int64_t>(q0) * a.qs[2]);
-    const char* dob = reinterpret_cast<const char*>(p.dout + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(q0) * a.os[2]);
+    const int64_t rows = a.Sq - q0;  // rows of the sequence from q0 on (>= 1)
+    const buffer_rsrc qb = make_buffer(a.q + b * a.qs[0] + hq * a.qs[1] + static_cast<int64_t>(q0) * a.qs[2],
+                                       ((rows - 1) * a.qs[2] + D) * 2);
+    const buffer_rsrc dob = make_buffer(p.dout + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(q0) * a.os[2],
+                                        ((rows - 1) * a.os[2] + D) * 2);
     const int64_t row0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + q0;
-    if (q0 + BM <= a.Sq) {
+    const buffer_rsrc lb = make_buffer(p.lse + row0, rows * 4);
+    const buffer_rsrc db = make_buffer(p.delta + row0, rows * 4);
 #pragma unroll
-      for (int i = 0; i < C::kQLoads; ++i) {
-        qreg[i] = *reinterpret_cast<const u32x4*>(qb + q_off[i]);
-        doreg[i] = *reinterpret_cast<const u32x4*>(dob + do_off[i]);
-      }
-      lreg = p.lse[row0 + tid % BM];
-      dreg = p.delta[row0 + tid % BM];
-    } else {
-      const int last = a.Sq - 1 - q0;  // last live row of the tile
-#pragma unroll
-      for (int i = 0; i < C::kQLoads; ++i) {
-        const int idx = tid + i * C::kThreads;
-        const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-        const int rc = r < last ? r : last;
-        qreg[i] = *reinterpret_cast<const u32x4*>(qb + (static_cast<int64_t>(rc) * a.qs[2] + cv * 8) * 2);
-        doreg[i] = *reinterpret_cast<const u32x4*>(dob + (static_cast<int64_t>(rc) * a.os[2] + cv * 8) * 2);
-      }
-      const int rl = (tid % BM) < last ? (tid % BM) : last;
-      lreg = p.lse[row0 + rl];
-      dreg = p.delta[row0 + rl];
+    for (int i = 0; i < C::kQLoads; ++i) {
+      qreg[i] = buffer_load_b128(qb, q_off[i]);
+      doreg[i] = buffer_load_b128(dob, do_off[i]);
     }
+    lreg = buffer_load_f32(lb, row_off);
+    dreg = buffer_load_f32(db, row_off);
   };
   auto stage = [&](int it, int buf) {
     const int q0 = (qt_start + it % tiles_per_head) * BM;
@@ -153,38 +144,37 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     __bf16* sdO = sQ + BM * LDQ;
     float* sL = reinterpret_cast<float*>(sdO + BM * LDQ);
     float* sDelta = sL + BM;
-    const bool full = q0 + BM <= a.Sq;
 #pragma unroll
     for (int i = 0; i < C::kQLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      u32x4 qv = qreg[i], dv4 = doreg[i];
-      if (!full && q0 + r >= a.Sq) { qv = u32x4{0, 0, 0, 0}; dv4 = u32x4{0, 0, 0, 0}; }
-      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = qv;
-      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = dv4;
+      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = qreg[i];
+      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = doreg[i];
     }
     if (tid < BM) {
       // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
       const bool live = q0 + tid < a.Sq && lreg != -INFINITY;
       sL[tid] = live ? lreg * kLog2e : INFINITY;
-      sDelta[tid] = live ? -dreg : 0.f;   // stored negated: it is loaded straight into the dP accumulator
+      sDelta[tid] = -dreg;   // stored negated: it is loaded straight into the dP accumulator (0 past Sq)
     }
   };
 
   if (n_iter > 0) {
     prefetch(0);
     stage(0, 0);
-    if (n_iter > 1) prefetch(1);
   }
+  // The K / V fragment loads above are complete by now on every path that enters the loop (the LDS fill
+  // waited for all loads), but not on the static path that skips the fill; saying so here keeps the compiler
+  // from putting a vmcnt(0) wait in front of the loop's first MFMAs, where it would wait for the prefetch
+  // of the NEXT tile on every trip.
+  __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
   __syncthreads();
 
   const int kw0 = key0 + 32 * wave;
   for (int it = 0; it < n_iter; ++it) {
-    // stage tile it+1 into the other buffer (its readers finished before the barrier that ended trip it-1)
-    if (it + 1 < n_iter) {
-      stage(it + 1, (it + 1) & 1);
-      if (it + 2 < n_iter) prefetch(it + 2);
-    }
+    // tile it+1 travels global -> registers while this trip computes; it goes to the other LDS buffer at
+    // the end of the trip (that buffer's readers finished before the barrier that ended trip it-1)
+    if (it + 1 < n_iter) prefetch(it + 1);
     const int q0 = (qt_start + it % tiles_per_head) * BM;
     const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + (it & 1) * C::kBufBytes);
     const __bf16* sdO = sQ + BM * LDQ;
@@ -249,6 +239,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
         }
       }
     }
+    if (it + 1 < n_iter) stage(it + 1, (it + 1) & 1);
     __syncthreads();  // all waves are done with buffer it&1 (refilled in trip it+1) and tile it+1 is visible
   }
 
@@ -381,43 +372,54 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
   }
   const int ntiles = (kv_end + KT - 1) / KT;
 
+  // K / V tiles travel global -> registers -> LDS with buffer loads (wave-uniform resource per tile, per-lane
+  // byte offsets computed once, rows past Sk read as zeros)
   u32x4 kreg[C::kLoads], vreg[C::kLoads];
+  uint32_t k_off[C::kLoads], v_off[C::kLoads];
+#pragma unroll
+  for (int i = 0; i < C::kLoads; ++i) {
+    const int idx = tid + i * C::kThreads;
+    const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+    k_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.ks[2] + cv * 8) * 2);
+    v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
+  }
   auto load_tile = [&](int k0) {
+    const int64_t rows = a.Sk - k0;  // >= 1 for every tile the loop visits
+    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], ((rows - 1) * a.ks[2] + D) * 2);
+    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], ((rows - 1) * a.vs[2] + D) * 2);
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
-      const int idx = tid + i * C::kThreads;
-      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const int key = (k0 + r < a.Sk) ? k0 + r : a.Sk - 1;
-      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + cv * 8);
-      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + cv * 8);
+      kreg[i] = buffer_load_b128(kb, k_off[i]);
+      vreg[i] = buffer_load_b128(vb, v_off[i]);
     }
   };
-  auto store_tile = [&](int k0, int buf) {
+  auto store_tile = [&](int buf) {
     __bf16* sK = smem + buf * C::kTileElems;
     __bf16* sV = sK + KT * LDK;
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const bool live = k0 + r < a.Sk;
-      const u32x4 zero = {0, 0, 0, 0};
-      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = live ? kreg[i] : zero;
-      *reinterpret_cast<u32x4*>(&sV[r * LDK + cv * 8]) = live ? vreg[i] : zero;
+      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = kreg[i];
+      *reinterpret_cast<u32x4*>(&sV[r * LDK + cv * 8]) = vreg[i];
     }
   };
 
   if (ntiles > 0) {
     load_tile(0);
-    store_tile(0, 0);
-    if (ntiles > 1) load_tile(KT);
+    store_tile(0);
   }
+  // all loads so far are complete on every path into the loop (the LDS fill waited for the newest); stating
+  // it keeps a vmcnt(0) wait, which would hit the next tile's prefetch, out of the loop body
+  __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
+  if (ntiles > 1) load_tile(KT);
   __syncthreads();
 
   const int blk_q_lo = a.q_offset + q0 + wave * 32;  // position of this wave's first query
   const int qpos = a.q_offset + qrow;
   for (int t = 0; t < ntiles; ++t) {
     if (t + 1 < ntiles) {
-      store_tile((t + 1) * KT, (t + 1) & 1);
+      store_tile((t + 1) & 1);
       if (t + 2 < ntiles) load_tile((t + 2) * KT);
     }
     const __bf16* sK = smem + (t & 1) * C::kTileElems;

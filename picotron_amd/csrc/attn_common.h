@@ -44,6 +44,25 @@ __device__ __forceinline__ bf16x8 lds_read_tr_pair(const __bf16* p, int ld) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// s_waitcnt immediate for "vmcnt(0)" with the other counters left at their maxima (gfx9 encoding:
+// vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14])
+constexpr int kWaitVmcnt0 = 0x0F70;
+
+// ---- buffer loads.  A buffer resource (4 SGPRs: base, byte count) plus a 32-bit per-lane byte offset replaces
+// 64-bit per-lane addresses; a lane whose offset is past the byte count reads zeros, which is how tile rows
+// past the end of a sequence become zero rows without clamps or selects.
+using buffer_rsrc = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ buffer_rsrc make_buffer(const void* base, int64_t bytes) {
+  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0xffffffffll ? 0xffffffffu : static_cast<uint32_t>(bytes));
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(n), 0x00020000);
+}
+__device__ __forceinline__ u32x4 buffer_load_b128(buffer_rsrc r, uint32_t byte_off) {
+  return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(byte_off), 0, 0));
+}
+__device__ __forceinline__ float buffer_load_f32(buffer_rsrc r, uint32_t byte_off) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, static_cast<int>(byte_off), 0, 0));
+}
+
 __device__ __forceinline__ bf16x8 pack8(const f32x16& c, int base) {
   bf16x8 r;
 #pragma unroll

@@ -124,45 +124,57 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   }
   const int ntiles = (kv_end + KT - 1) / KT;
 
-  // ---- global -> register -> LDS staging of one K/V tile of KT keys.  Loads are unconditional (rows
-  //      past Sk are clamped and zeroed on the way into LDS) so the loop body holds no wait for memory
-  //      other than the one in front of the LDS fill, a whole tile after the loads were issued.
+  // ---- global -> register -> LDS staging of one K/V tile of KT keys, with buffer loads: a wave-uniform
+  //      resource per tile (first key row, bytes left in the sequence) plus per-lane byte offsets that are
+  //      computed once; rows past Sk read as zeros.  The loop body holds no wait for memory other than the
+  //      one in front of the LDS fill, a whole tile after the loads were issued.
   u32x4 kreg[C::kLoads], vreg[C::kLoads];
+  uint32_t k_off[C::kLoads], v_off[C::kLoads];
+#pragma unroll
+  for (int i = 0; i < C::kLoads; ++i) {
+    const int idx = tid + i * C::kThreads;
+    const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
+    k_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.ks[2] + cv * 8) * 2);
+    v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
+  }
   auto load_tile = [&](int k0) {
+    const int64_t rows = a.Sk - k0;  // >= 1 for every tile the loop visits
+    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], ((rows - 1) * a.ks[2] + D) * 2);
+    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], ((rows - 1) * a.vs[2] + D) * 2);
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
-      const int idx = tid + i * C::kThreads;
-      const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const int key = (k0 + r < a.Sk) ? k0 + r : a.Sk - 1;
-      kreg[i] = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + cv * 8);
-      vreg[i] = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + cv * 8);
+      kreg[i] = buffer_load_b128(kb, k_off[i]);
+      vreg[i] = buffer_load_b128(vb, v_off[i]);
     }
   };
-  auto store_tile = [&](int k0, int buf) {
+  auto store_tile = [&](int buf) {
     __bf16* sK = smem + buf * C::kTileElems;
     __bf16* sV = sK + KT * LDK;
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      const bool live = k0 + r < a.Sk;
-      const u32x4 zero = {0, 0, 0, 0};
-      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = live ? kreg[i] : zero;
-      *reinterpret_cast<u32x4*>(&sV[r * LDV + cv * 8]) = live ? vreg[i] : zero;
+      *reinterpret_cast<u32x4*>(&sK[r * LDK + cv * 8]) = kreg[i];
+      *reinterpret_cast<u32x4*>(&sV[r * LDV + cv * 8]) = vreg[i];
     }
   };
 
   if (ntiles > 0) {
     load_tile(0);
-    store_tile(0, 0);
-    if (ntiles > 1) load_tile(KT);
+    store_tile(0);
   }
+  // Every load issued so far (Q fragments, the merge state, tile 0) is complete on each path that enters the
+  // loop, because the LDS fill waited for the newest of them -- but not on the static path that skips the
+  // fill.  Saying so here keeps the compiler from putting a vmcnt(0) wait in front of the loop's first MFMAs,
+  // where it would wait for the prefetch of the NEXT tile on every trip.
+  __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
+  if (ntiles > 1) load_tile(KT);
   __syncthreads();
 
   for (int t = 0; t < ntiles; ++t) {
     // stage tile t+1 into the other buffer (its readers finished before the barrier that ended trip t-1)
     if (t + 1 < ntiles) {
-      store_tile((t + 1) * KT, (t + 1) & 1);
+      store_tile((t + 1) & 1);
       if (t + 2 < ntiles) load_tile((t + 2) * KT);
     }
     const __bf16* sK = smem + (t & 1) * C::kTileElems;
