@@ -159,7 +159,7 @@ int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* dout, const
  * dq:     [B,Hq,Sq,D] addressed by dq_stride (element strides for b, h, s, multiples of 4; NULL = contiguous);
  *         dq_dtype PICO_F32 with dq_accumulate = 1 adds into the buffer (the running sum over ring steps),
  *         dq_accumulate = 0 overwrites; PICO_BF16 overwrites.
- * dk, dv: [B,Hkv,Sk,D] addressed by dkv_stride (NULL = contiguous); same dtype / accumulate rules (the
+ * dk, dv: [B,Hkv,Sk,D] addressed by dkv_stride (multiples of 8; NULL = contiguous); same dtype / accumulate rules (the
  *         travelling fp32 accumulators of the ring).  With Hq > Hkv the group's query heads are reduced
  *         inside the kernel.
  * A gradient that is not wanted is passed as NULL (dq, or dk and dv together) and its kernel is skipped.

@@ -48,7 +48,9 @@ struct KvCfg {
   static constexpr int kQLoads = BM * kVecPerRow / kThreads;
   static constexpr int kBufElems = 2 * BM * LDQ;                       // Q + dO tile of one stage (bf16)
   static constexpr size_t kBufBytes = kBufElems * sizeof(__bf16) + 2 * BM * sizeof(float);
+  static constexpr size_t kEpiBytes = 32 * (D * 4 + 16);               // one wave's rows in the epilogue (fp32 case)
   static constexpr size_t kLdsBytes = 2 * kBufBytes;                   // double-buffered
+  static_assert(NW * kEpiBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
 };
 
 template <int D>
@@ -104,10 +106,11 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
   const int tiles_per_head = n_qtiles > qt_start ? n_qtiles - qt_start : 0;
   const int n_iter = tiles_per_head * group;
 
-  // Global -> register prefetch of a Q / dO tile (+ lse, delta) with buffer loads: the resource is rebuilt
-  // per tile from wave-uniform values (head, first row, rows left in the sequence), the per-lane byte
-  // offsets are computed once, and rows past Sq read as zeros.  Nothing here uses a loaded value, so the
-  // loop holds no wait for memory other than the one in front of the LDS fill, a whole trip after the loads.
+  // Global -> register prefetch of a Q / dO tile (+ lse, delta) with buffer loads.  A cursor (wave-uniform:
+  // it lives in scalar registers) walks the trip space; stepping to the next tile of the same head is a few
+  // scalar adds, only a change of head recomputes addresses.  The per-lane byte offsets are computed once,
+  // and rows past Sq read as zeros because they lie past the end of the buffer window.  Every instruction
+  // of a wave costs an issue slot, scalar ones included, so the per-trip bookkeeping is kept this small.
   u32x4 qreg[C::kQLoads], doreg[C::kQLoads];
   float lreg = 0.f, dreg = 0.f;
   uint32_t q_off[C::kQLoads], do_off[C::kQLoads];
@@ -119,17 +122,39 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     do_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.os[2] + cv * 8) * 2);
   }
   const uint32_t row_off = static_cast<uint32_t>((tid % BM) * 4);
-  auto prefetch = [&](int it) {
-    const int hq = hkv * group + it / tiles_per_head;
-    const int q0 = (qt_start + it % tiles_per_head) * BM;
-    const int64_t rows = a.Sq - q0;  // rows of the sequence from q0 on (>= 1)
-    const buffer_rsrc qb = make_buffer(a.q + b * a.qs[0] + hq * a.qs[1] + static_cast<int64_t>(q0) * a.qs[2],
-                                       ((rows - 1) * a.qs[2] + D) * 2);
-    const buffer_rsrc dob = make_buffer(p.dout + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(q0) * a.os[2],
-                                        ((rows - 1) * a.os[2] + D) * 2);
-    const int64_t row0 = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + q0;
-    const buffer_rsrc lb = make_buffer(p.lse + row0, rows * 4);
-    const buffer_rsrc db = make_buffer(p.delta + row0, rows * 4);
+  const uint32_t q_step = static_cast<uint32_t>(BM * a.qs[2] * 2), do_step = static_cast<uint32_t>(BM * a.os[2] * 2);
+  struct Cursor {
+    int tile, head;                  // query tile within the head, query head
+    const char *q, *dout;            // first row of the tile
+    const float *lse, *delta;
+    uint32_t q_left, do_left, rows_left;  // bytes from there to the end of the head's rows
+  } cur;
+  auto seek = [&](int head, int tile) {
+    const int q0 = tile * BM;
+    cur.tile = tile;
+    cur.head = head;
+    cur.q = reinterpret_cast<const char*>(a.q + b * a.qs[0] + head * a.qs[1] + static_cast<int64_t>(q0) * a.qs[2]);
+    cur.dout = reinterpret_cast<const char*>(p.dout + b * a.os[0] + head * a.os[1] + static_cast<int64_t>(q0) * a.os[2]);
+    const int64_t row0 = (static_cast<int64_t>(b) * a.Hq + head) * a.Sq + q0;
+    cur.lse = p.lse + row0;
+    cur.delta = p.delta + row0;
+    cur.q_left = span_bytes(a.Sq - q0, a.qs[2], D);
+    cur.do_left = span_bytes(a.Sq - q0, a.os[2], D);
+    cur.rows_left = static_cast<uint32_t>(a.Sq - q0) * 4u;
+  };
+  auto advance = [&]() {
+    if (cur.tile + 1 == n_qtiles) {
+      seek(cur.head + 1, qt_start);
+    } else {
+      ++cur.tile;
+      cur.q += q_step;  cur.q_left -= q_step;
+      cur.dout += do_step;  cur.do_left -= do_step;
+      cur.lse += BM;  cur.delta += BM;  cur.rows_left -= BM * 4;
+    }
+  };
+  auto prefetch = [&]() {  // the tile under the cursor
+    const buffer_rsrc qb = make_buffer(cur.q, cur.q_left), dob = make_buffer(cur.dout, cur.do_left);
+    const buffer_rsrc lb = make_buffer(cur.lse, cur.rows_left), db = make_buffer(cur.delta, cur.rows_left);
 #pragma unroll
     for (int i = 0; i < C::kQLoads; ++i) {
       qreg[i] = buffer_load_b128(qb, q_off[i]);
@@ -138,8 +163,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     lreg = buffer_load_f32(lb, row_off);
     dreg = buffer_load_f32(db, row_off);
   };
-  auto stage = [&](int it, int buf) {
-    const int q0 = (qt_start + it % tiles_per_head) * BM;
+  auto stage = [&](int buf) {  // the prefetched tile (still under the cursor) goes to LDS buffer `buf`
     __bf16* sQ = reinterpret_cast<__bf16*>(smem_raw + buf * C::kBufBytes);
     __bf16* sdO = sQ + BM * LDQ;
     float* sL = reinterpret_cast<float*>(sdO + BM * LDQ);
@@ -153,15 +177,16 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     }
     if (tid < BM) {
       // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
-      const bool live = q0 + tid < a.Sq && lreg != -INFINITY;
+      const bool live = static_cast<uint32_t>(tid) * 4u < cur.rows_left && lreg != -INFINITY;
       sL[tid] = live ? lreg * kLog2e : INFINITY;
       sDelta[tid] = -dreg;   // stored negated: it is loaded straight into the dP accumulator (0 past Sq)
     }
   };
 
   if (n_iter > 0) {
-    prefetch(0);
-    stage(0, 0);
+    seek(hkv * group, qt_start);
+    prefetch();
+    stage(0);
   }
   // The K / V fragment loads above are complete by now on every path that enters the loop (the LDS fill
   // waited for all loads), but not on the static path that skips the fill; saying so here keeps the compiler
@@ -171,12 +196,18 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
   __syncthreads();
 
   const int kw0 = key0 + 32 * wave;
+  int tile = qt_start;       // query tile (within its head) of the trip being computed
+  uint32_t buf_off = 0;      // byte offset of the LDS buffer being read
   for (int it = 0; it < n_iter; ++it) {
     // tile it+1 travels global -> registers while this trip computes; it goes to the other LDS buffer at
     // the end of the trip (that buffer's readers finished before the barrier that ended trip it-1)
-    if (it + 1 < n_iter) prefetch(it + 1);
-    const int q0 = (qt_start + it % tiles_per_head) * BM;
-    const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + (it & 1) * C::kBufBytes);
+    const bool has_next = it + 1 < n_iter;
+    if (has_next) {
+      advance();
+      prefetch();
+    }
+    const int q0 = tile * BM;
+    const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + buf_off);
     const __bf16* sdO = sQ + BM * LDQ;
     const float* sL = reinterpret_cast<const float*>(sdO + BM * LDQ);
     const float* sDelta = sL + BM;
@@ -234,53 +265,80 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
           const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
           const bf16x8 dof = lds_read_tr_pair(&sdO[qr * LDQ + col], LDQ);
           const bf16x8 qf = lds_read_tr_pair(&sQ[qr * LDQ + col], LDQ);
-          dv_acc[db] = mfma32(pf, dof, dv_acc[db]);
-          dk_acc[db] = mfma32(dsf, qf, dk_acc[db]);
+          // transposed products dV^T = dO^T P and dK^T = Q^T dS: lane = key, registers = 4 consecutive d,
+          // which is what lets the epilogue write whole 16-byte pieces of a row
+          dv_acc[db] = mfma32(dof, pf, dv_acc[db]);
+          dk_acc[db] = mfma32(qf, dsf, dk_acc[db]);
         }
       }
     }
-    if (it + 1 < n_iter) stage(it + 1, (it + 1) & 1);
-    __syncthreads();  // all waves are done with buffer it&1 (refilled in trip it+1) and tile it+1 is visible
+    buf_off ^= static_cast<uint32_t>(C::kBufBytes);
+    if (has_next) stage(buf_off != 0);
+    tile = tile + 1 == n_qtiles ? qt_start : tile + 1;
+    __syncthreads();  // all waves are done with the buffer just read (refilled in the next trip) and the next tile is visible
   }
 
-  // ---- epilogue: dK (scaled) and dV rows of this wave's keys.  In accumulate mode all reads of a block
-  //      are issued before the first write so they overlap instead of serialising on memory latency.
-#pragma unroll
-  for (int db = 0; db < D / 32; ++db) {
-    int64_t off[16];
-    bool live[16];
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int key = key0 + 32 * wave + 8 * (i / 4) + 4 * h + (i % 4);
-      live[i] = key < a.Sk;
-      off[i] = b * p.dks[0] + hkv * p.dks[1] + static_cast<int64_t>(live[i] ? key : 0) * p.dks[2] + 32 * db + n;
-    }
+  // ---- epilogue: dK (scaled) and dV rows of this wave's 32 keys.  Each wave turns its accumulators
+  //      (lane = key, registers 4j..4j+3 = d columns 32db + 8j + 4h ..+3) into rows in its own piece of
+  //      LDS -- free now: the loop ended on a barrier -- and writes them out 16 bytes per lane, whole
+  //      128-byte lines at a time.  In accumulate mode all reads are issued before the first write.
+  unsigned char* region = smem_raw + wave * C::kEpiBytes;
+  const int64_t out_base = b * p.dks[0] + hkv * p.dks[1];
+  auto flush = [&](const f32x16 (&acc)[D / 32], float scale, void* dst) {
     if (p.dkv_f32) {
-      float* pk = static_cast<float*>(p.dk);
-      float* pv = static_cast<float*>(p.dv);
-      float ok[16], ov[16];
+      constexpr int kPitch = D * 4 + 16, kChunks = D / 4, kPerLane = 32 * kChunks / 64;
 #pragma unroll
-      for (int i = 0; i < 16; ++i) { ok[i] = 0.f; ov[i] = 0.f; }
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          f32x4 v4;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) v4[t] = acc[db][4 * j + t] * scale;
+          *reinterpret_cast<f32x4*>(region + n * kPitch + (32 * db + 8 * j + 4 * h) * 4) = v4;
+        }
+      float* g[kPerLane];
+      f32x4 v[kPerLane], old[kPerLane];
+#pragma unroll
+      for (int t = 0; t < kPerLane; ++t) {
+        const int idx = lane + 64 * t, r = idx / kChunks, ch = idx % kChunks;
+        const int key = key0 + 32 * wave + r;
+        v[t] = *reinterpret_cast<const f32x4*>(region + r * kPitch + ch * 16);
+        g[t] = key < a.Sk ? static_cast<float*>(dst) + out_base + static_cast<int64_t>(key) * p.dks[2] + ch * 4 : nullptr;
+        old[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
       if (p.dkv_accumulate) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i)
-          if (live[i]) { ok[i] = pk[off[i]]; ov[i] = pv[off[i]]; }
+        for (int t = 0; t < kPerLane; ++t)
+          if (g[t]) old[t] = *reinterpret_cast<const f32x4*>(g[t]);
       }
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (live[i]) {
-          pk[off[i]] = ok[i] + dk_acc[db][i] * a.sm_scale;
-          pv[off[i]] = ov[i] + dv_acc[db][i];
-        }
+      for (int t = 0; t < kPerLane; ++t)
+        if (g[t]) *reinterpret_cast<f32x4*>(g[t]) = v[t] + old[t];
     } else {
+      constexpr int kPitch = D * 2 + 16, kChunks = D / 8, kPerLane = 32 * kChunks / 64;
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        if (live[i]) {
-          static_cast<__bf16*>(p.dk)[off[i]] = static_cast<__bf16>(dk_acc[db][i] * a.sm_scale);
-          static_cast<__bf16*>(p.dv)[off[i]] = static_cast<__bf16>(dv_acc[db][i]);
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          bf16x4 v4;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) v4[t] = static_cast<__bf16>(acc[db][4 * j + t] * scale);
+          *reinterpret_cast<bf16x4*>(region + n * kPitch + (32 * db + 8 * j + 4 * h) * 2) = v4;
         }
+#pragma unroll
+      for (int t = 0; t < kPerLane; ++t) {
+        const int idx = lane + 64 * t, r = idx / kChunks, ch = idx % kChunks;
+        const int key = key0 + 32 * wave + r;
+        const u32x4 v = *reinterpret_cast<const u32x4*>(region + r * kPitch + ch * 16);
+        // streaming store: nothing on this GPU reads the bf16 gradients back soon, and lines that stay dirty
+        // in L2 are only written back when the kernel ends
+        if (key < a.Sk)
+          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(static_cast<__bf16*>(dst) + out_base + static_cast<int64_t>(key) * p.dks[2] + ch * 8));
+      }
     }
-  }
+  };
+  flush(dk_acc, a.sm_scale, p.dk);
+  flush(dv_acc, 1.f, p.dv);
 }
 
 // D = 64 fits two workgroups per CU (<= 256 registers per lane), which lets one workgroup's MFMA
@@ -384,9 +442,8 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
   }
   auto load_tile = [&](int k0) {
-    const int64_t rows = a.Sk - k0;  // >= 1 for every tile the loop visits
-    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], ((rows - 1) * a.ks[2] + D) * 2);
-    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], ((rows - 1) * a.vs[2] + D) * 2);
+    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], span_bytes(a.Sk - k0, a.ks[2], D));
+    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], span_bytes(a.Sk - k0, a.vs[2], D));
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       kreg[i] = buffer_load_b128(kb, k_off[i]);
@@ -630,8 +687,8 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
   if (((have_q || have_k) && desc->Sq > 0 && (!q || !dout || !lse || !delta)) ||
       ((have_q || have_k) && desc->Sk > 0 && (!k || !v)))
     return fail(PICO_ERR_NULL, "pico_attn_bwd: q, k, v, dout, lse and delta are required");
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq))
-    return fail(PICO_ERR_ALIGN, "pico_attn_bwd: q, k, v, dout and dq must be 16-byte aligned");
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
+    return fail(PICO_ERR_ALIGN, "pico_attn_bwd: q, k, v, dout, dq, dk and dv must be 16-byte aligned");
   BwdParams p;
   p.a = make_params(desc, q, k, v);
   p.dout = static_cast<const __bf16*>(dout);
@@ -653,8 +710,8 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
     }
     return true;
   };
-  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, 4) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 1))
-    return fail(PICO_ERR_STRIDE, "pico_attn_bwd: dq strides must be non-negative multiples of 4, dk/dv strides non-negative");
+  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, 4) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 8))
+    return fail(PICO_ERR_STRIDE, "pico_attn_bwd: dq strides must be non-negative multiples of 4, dk/dv strides non-negative multiples of 8");
   hipStream_t s = static_cast<hipStream_t>(stream);
   int rc = PICO_OK;
   if (have_k) {

@@ -52,9 +52,13 @@ constexpr int kWaitVmcnt0 = 0x0F70;
 // 64-bit per-lane addresses; a lane whose offset is past the byte count reads zeros, which is how tile rows
 // past the end of a sequence become zero rows without clamps or selects.
 using buffer_rsrc = __amdgpu_buffer_rsrc_t;
-__device__ __forceinline__ buffer_rsrc make_buffer(const void* base, int64_t bytes) {
-  const uint32_t n = bytes <= 0 ? 0u : (bytes > 0xffffffffll ? 0xffffffffu : static_cast<uint32_t>(bytes));
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(n), 0x00020000);
+// `bytes` is the exact size of the window: the entry points reject tensors whose rows of one head span 4 GiB or more
+__device__ __forceinline__ buffer_rsrc make_buffer(const void* base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), 0x00020000);
+}
+// bytes from the first element of row 0 to the end of row rows-1, for rows of D bf16 elements `stride` elements apart
+__device__ __forceinline__ uint32_t span_bytes(int rows, int64_t stride, int D) {
+  return rows <= 0 ? 0u : static_cast<uint32_t>((static_cast<int64_t>(rows - 1) * stride + D) * 2);
 }
 __device__ __forceinline__ u32x4 buffer_load_b128(buffer_rsrc r, uint32_t byte_off) {
   return __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(r, static_cast<int>(byte_off), 0, 0));

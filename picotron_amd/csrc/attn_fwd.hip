@@ -138,9 +138,8 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
   }
   auto load_tile = [&](int k0) {
-    const int64_t rows = a.Sk - k0;  // >= 1 for every tile the loop visits
-    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], ((rows - 1) * a.ks[2] + D) * 2);
-    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], ((rows - 1) * a.vs[2] + D) * 2);
+    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], span_bytes(a.Sk - k0, a.ks[2], D));
+    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], span_bytes(a.Sk - k0, a.vs[2], D));
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       kreg[i] = buffer_load_b128(kb, k_off[i]);
@@ -328,6 +327,12 @@ int check_attn_desc(const char* fn, const pico_attn_desc* d) {
     for (int i = 0; i < 3; ++i)
       if (st[i] < 0 || st[i] % 8 != 0)
         return fail(PICO_ERR_STRIDE, "%s: strides must be non-negative multiples of 8 elements", fn);
+  // the kernels address one head's rows through 32-bit byte offsets
+  const int64_t spans[4] = {(d->Sq - 1) * d->q_stride[2], (d->Sk - 1) * d->k_stride[2], (d->Sk - 1) * d->v_stride[2],
+                            (d->Sq - 1) * d->o_stride[2]};
+  for (int64_t span : spans)
+    if ((span + d->D) * 2 >= (1LL << 32))
+      return fail(PICO_ERR_STRIDE, "%s: the rows of one head must span less than 4 GiB", fn);
   return PICO_OK;
 }
 
