@@ -48,9 +48,8 @@ struct KvCfg {
   static constexpr int kQLoads = BM * kVecPerRow / kThreads;
   static constexpr int kBufElems = 2 * BM * LDQ;                       // Q + dO tile of one stage (bf16)
   static constexpr size_t kBufBytes = kBufElems * sizeof(__bf16) + 2 * BM * sizeof(float);
-  static constexpr size_t kEpiBytes = 32 * (D * 4 + 16);               // one wave's rows in the epilogue (fp32 case)
   static constexpr size_t kLdsBytes = 2 * kBufBytes;                   // double-buffered
-  static_assert(NW * kEpiBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
+  static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
 };
 
 template <int D>
@@ -278,67 +277,22 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
     __syncthreads();  // all waves are done with the buffer just read (refilled in the next trip) and the next tile is visible
   }
 
-  // ---- epilogue: dK (scaled) and dV rows of this wave's 32 keys.  Each wave turns its accumulators
-  //      (lane = key, registers 4j..4j+3 = d columns 32db + 8j + 4h ..+3) into rows in its own piece of
-  //      LDS -- free now: the loop ended on a barrier -- and writes them out 16 bytes per lane, whole
-  //      128-byte lines at a time.  In accumulate mode all reads are issued before the first write.
-  unsigned char* region = smem_raw + wave * C::kEpiBytes;
-  const int64_t out_base = b * p.dks[0] + hkv * p.dks[1];
-  auto flush = [&](const f32x16 (&acc)[D / 32], float scale, void* dst) {
+  // ---- epilogue: dK (scaled) and dV rows of this wave's 32 keys, through the wave's piece of LDS (free now:
+  //      the loop ended on a barrier).  bf16 gradients are written with streaming stores: nothing on this
+  //      GPU reads them back soon, and lines left dirty in L2 are only written back when the kernel ends.
+  {
+    unsigned char* region = smem_raw + wave * kRowRegionBytes;
+    const int row0 = key0 + 32 * wave;
+    const int rows_live = a.Sk - row0;
+    const int64_t off = b * p.dks[0] + hkv * p.dks[1] + static_cast<int64_t>(row0) * p.dks[2];
     if (p.dkv_f32) {
-      constexpr int kPitch = D * 4 + 16, kChunks = D / 4, kPerLane = 32 * kChunks / 64;
-#pragma unroll
-      for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          f32x4 v4;
-#pragma unroll
-          for (int t = 0; t < 4; ++t) v4[t] = acc[db][4 * j + t] * scale;
-          *reinterpret_cast<f32x4*>(region + n * kPitch + (32 * db + 8 * j + 4 * h) * 4) = v4;
-        }
-      float* g[kPerLane];
-      f32x4 v[kPerLane], old[kPerLane];
-#pragma unroll
-      for (int t = 0; t < kPerLane; ++t) {
-        const int idx = lane + 64 * t, r = idx / kChunks, ch = idx % kChunks;
-        const int key = key0 + 32 * wave + r;
-        v[t] = *reinterpret_cast<const f32x4*>(region + r * kPitch + ch * 16);
-        g[t] = key < a.Sk ? static_cast<float*>(dst) + out_base + static_cast<int64_t>(key) * p.dks[2] + ch * 4 : nullptr;
-        old[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-      if (p.dkv_accumulate) {
-#pragma unroll
-        for (int t = 0; t < kPerLane; ++t)
-          if (g[t]) old[t] = *reinterpret_cast<const f32x4*>(g[t]);
-      }
-#pragma unroll
-      for (int t = 0; t < kPerLane; ++t)
-        if (g[t]) *reinterpret_cast<f32x4*>(g[t]) = v[t] + old[t];
+      wave_store_rows<D, true>(region, dk_acc, a.sm_scale, static_cast<float*>(p.dk) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
+      wave_store_rows<D, true>(region, dv_acc, 1.f, static_cast<float*>(p.dv) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
     } else {
-      constexpr int kPitch = D * 2 + 16, kChunks = D / 8, kPerLane = 32 * kChunks / 64;
-#pragma unroll
-      for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          bf16x4 v4;
-#pragma unroll
-          for (int t = 0; t < 4; ++t) v4[t] = static_cast<__bf16>(acc[db][4 * j + t] * scale);
-          *reinterpret_cast<bf16x4*>(region + n * kPitch + (32 * db + 8 * j + 4 * h) * 2) = v4;
-        }
-#pragma unroll
-      for (int t = 0; t < kPerLane; ++t) {
-        const int idx = lane + 64 * t, r = idx / kChunks, ch = idx % kChunks;
-        const int key = key0 + 32 * wave + r;
-        const u32x4 v = *reinterpret_cast<const u32x4*>(region + r * kPitch + ch * 16);
-        // streaming store: nothing on this GPU reads the bf16 gradients back soon, and lines that stay dirty
-        // in L2 are only written back when the kernel ends
-        if (key < a.Sk)
-          __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(static_cast<__bf16*>(dst) + out_base + static_cast<int64_t>(key) * p.dks[2] + ch * 8));
-      }
+      wave_store_rows<D, false>(region, dk_acc, a.sm_scale, static_cast<__bf16*>(p.dk) + off, p.dks[2], rows_live, lane, false, true);
+      wave_store_rows<D, false>(region, dv_acc, 1.f, static_cast<__bf16*>(p.dv) + off, p.dks[2], rows_live, lane, false, true);
     }
-  };
-  flush(dk_acc, a.sm_scale, p.dk);
-  flush(dv_acc, 1.f, p.dv);
+  }
 }
 
 // D = 64 fits two workgroups per CU (<= 256 registers per lane), which lets one workgroup's MFMA
@@ -363,6 +317,7 @@ struct DqCfg {
   static constexpr int kLoads = KT * kVecPerRow / kThreads;
   static constexpr int kTileElems = 2 * KT * LDK;
   static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);  // double-buffered
+  static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
@@ -441,14 +396,20 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     k_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.ks[2] + cv * 8) * 2);
     v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
   }
-  auto load_tile = [&](int k0) {
-    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], span_bytes(a.Sk - k0, a.ks[2], D));
-    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], span_bytes(a.Sk - k0, a.vs[2], D));
+  // a cursor walks the key tiles in order: stepping it is four scalar adds instead of 64-bit multiplies
+  const char* k_ptr = reinterpret_cast<const char*>(kbase);
+  const char* v_ptr = reinterpret_cast<const char*>(vbase);
+  uint32_t k_left = span_bytes(a.Sk, a.ks[2], D), v_left = span_bytes(a.Sk, a.vs[2], D);
+  const uint32_t k_step = static_cast<uint32_t>(KT * a.ks[2] * 2), v_step = static_cast<uint32_t>(KT * a.vs[2] * 2);
+  auto load_tile = [&]() {  // the next tile of KT keys
+    const buffer_rsrc kb = make_buffer(k_ptr, k_left), vb = make_buffer(v_ptr, v_left);
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       kreg[i] = buffer_load_b128(kb, k_off[i]);
       vreg[i] = buffer_load_b128(vb, v_off[i]);
     }
+    k_ptr += k_step;  k_left -= k_step;
+    v_ptr += v_step;  v_left -= v_step;
   };
   auto store_tile = [&](int buf) {
     __bf16* sK = smem + buf * C::kTileElems;
@@ -463,13 +424,13 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
   };
 
   if (ntiles > 0) {
-    load_tile(0);
+    load_tile();
     store_tile(0);
   }
   // all loads so far are complete on every path into the loop (the LDS fill waited for the newest); stating
   // it keeps a vmcnt(0) wait, which would hit the next tile's prefetch, out of the loop body
   __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
-  if (ntiles > 1) load_tile(KT);
+  if (ntiles > 1) load_tile();
   __syncthreads();
 
   const int blk_q_lo = a.q_offset + q0 + wave * 32;  // position of this wave's first query
@@ -477,7 +438,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
   for (int t = 0; t < ntiles; ++t) {
     if (t + 1 < ntiles) {
       store_tile((t + 1) & 1);
-      if (t + 2 < ntiles) load_tile((t + 2) * KT);
+      if (t + 2 < ntiles) load_tile();
     }
     const __bf16* sK = smem + (t & 1) * C::kTileElems;
     const __bf16* sV = sK + KT * LDK;
@@ -540,28 +501,16 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     __syncthreads();
   }
 
-  // ---- epilogue: lane = query, registers = 4 consecutive d per (db, j)
-  if (!qlive) return;
-  const int64_t off = b * p.dqs[0] + hq * p.dqs[1] + static_cast<int64_t>(qrow) * p.dqs[2];
-#pragma unroll
-  for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int d = 32 * db + 8 * j + 4 * h;
-      if (p.dq_f32) {
-        float* dst = static_cast<float*>(p.dq) + off + d;
-        f32x4 v4 = {0.f, 0.f, 0.f, 0.f};
-        if (p.dq_accumulate) v4 = *reinterpret_cast<const f32x4*>(dst);
-#pragma unroll
-        for (int t = 0; t < 4; ++t) v4[t] += dq[db][4 * j + t] * a.sm_scale;
-        *reinterpret_cast<f32x4*>(dst) = v4;
-      } else {
-        u32x2 v2;
-        v2[0] = pack_bf16x2(dq[db][4 * j] * a.sm_scale, dq[db][4 * j + 1] * a.sm_scale);
-        v2[1] = pack_bf16x2(dq[db][4 * j + 2] * a.sm_scale, dq[db][4 * j + 3] * a.sm_scale);
-        *reinterpret_cast<u32x2*>(static_cast<__bf16*>(p.dq) + off + d) = v2;
-      }
-    }
+  // ---- epilogue: the wave's 32 dQ rows leave through its piece of LDS as whole lines (the loop ended on a barrier)
+  {
+    unsigned char* region = smem_raw + wave * kRowRegionBytes;
+    const int row0 = q0 + wave * 32;
+    const int64_t off = b * p.dqs[0] + hq * p.dqs[1] + static_cast<int64_t>(row0) * p.dqs[2];
+    if (p.dq_f32)
+      wave_store_rows<D, true>(region, dq, a.sm_scale, static_cast<float*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, p.dq_accumulate, false);
+    else
+      wave_store_rows<D, false>(region, dq, a.sm_scale, static_cast<__bf16*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, false, true);
+  }
 }
 
 // delta[row] = sum_d dO * O, one 16-byte vector of each per lane, D/8 lanes per row.
@@ -710,8 +659,8 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
     }
     return true;
   };
-  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, 4) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 8))
-    return fail(PICO_ERR_STRIDE, "pico_attn_bwd: dq strides must be non-negative multiples of 4, dk/dv strides non-negative multiples of 8");
+  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, p.dq_f32 ? 4 : 8) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 8))
+    return fail(PICO_ERR_STRIDE, "pico_attn_bwd: dq strides must be non-negative multiples of 4 (fp32) or 8 (bf16), dk/dv strides of 8");
   hipStream_t s = static_cast<hipStream_t>(stream);
   int rc = PICO_OK;
   if (have_k) {

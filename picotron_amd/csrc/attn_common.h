@@ -84,6 +84,76 @@ __device__ __forceinline__ float half_sum(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// ---- writing a wave's 32 result rows.  The accumulators of the transposed products hold, per lane, one row
+// (lane % 32) and, in registers 4j..4j+3 of block db, columns 32db + 8j + 4h ..+3 (h = lane / 32).  Stored
+// straight from that layout a wave would touch 32 different 128-byte lines with 8 or 16 bytes each per
+// instruction; instead the rows take a detour through a 32 x 144-byte piece of LDS that belongs to the wave
+// (the caller guarantees that every wave of the workgroup is done with the tile buffers) and leave as whole
+// 128-byte lines, 16 bytes per lane.  One pass moves 128 bytes of every row: 32 fp32 or 64 bf16 columns.
+//   dst_row0: address of column 0 of the wave's first row; row_stride in elements; rows_live rows exist.
+//   accumulate (fp32 only) adds to what is there; all its reads are issued before the first write.
+//   streaming marks bf16 stores non-temporal (the data is not read again by the kernels that follow soon).
+constexpr int kRowRegionBytes = 32 * 144;
+template <int D, bool kF32>
+__device__ __forceinline__ void wave_store_rows(unsigned char* region, const f32x16 (&acc)[D / 32], float scale,
+                                                void* dst_row0, int64_t row_stride, int rows_live, int lane,
+                                                bool accumulate, bool streaming) {
+  constexpr int kPitch = 144;
+  constexpr int kColsPerPass = kF32 ? 32 : 64;
+  const int n = lane % 32, h = lane / 32;
+#pragma unroll
+  for (int c0 = 0; c0 < D; c0 += kColsPerPass) {
+#pragma unroll
+    for (int db = c0 / 32; db < (c0 + kColsPerPass) / 32; ++db)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int col = 32 * db + 8 * j + 4 * h - c0;
+        if constexpr (kF32) {
+          f32x4 v4;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) v4[t] = acc[db][4 * j + t] * scale;
+          *reinterpret_cast<f32x4*>(region + n * kPitch + col * 4) = v4;
+        } else {
+          bf16x4 v4;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) v4[t] = static_cast<__bf16>(acc[db][4 * j + t] * scale);
+          *reinterpret_cast<bf16x4*>(region + n * kPitch + col * 2) = v4;
+        }
+      }
+    // 32 rows x 8 pieces of 16 bytes = 4 pieces per lane; 8 consecutive lanes cover one row's line
+    unsigned char* g[4];
+    u32x4 v[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int idx = lane + 64 * t, r = idx / 8, ch = idx % 8;
+      v[t] = *reinterpret_cast<const u32x4*>(region + r * kPitch + ch * 16);
+      g[t] = r < rows_live ? static_cast<unsigned char*>(dst_row0) +
+                                 (static_cast<int64_t>(r) * row_stride + c0) * (kF32 ? 4 : 2) + ch * 16
+                           : nullptr;
+    }
+    if constexpr (kF32) {
+      f32x4 old[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) old[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (accumulate) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (g[t]) old[t] = *reinterpret_cast<const f32x4*>(g[t]);
+      }
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        if (g[t]) *reinterpret_cast<f32x4*>(g[t]) = __builtin_bit_cast(f32x4, v[t]) + old[t];
+    } else {
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        if (g[t]) {
+          if (streaming) __builtin_nontemporal_store(v[t], reinterpret_cast<u32x4*>(g[t]));
+          else *reinterpret_cast<u32x4*>(g[t]) = v[t];
+        }
+    }
+  }
+}
+
 struct AttnParams {
   const __bf16* q; const __bf16* k; const __bf16* v;
   int B, Hq, Hkv, Sq, Sk;

@@ -34,6 +34,7 @@ struct FwdCfg {
   static constexpr int kLoads = KT * kVecPerRow / kThreads;  // 16-byte loads per thread per tensor
   static constexpr int kTileElems = KT * (LDK + LDV);
   static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);
+  static_assert(NW * QB * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
@@ -137,14 +138,20 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     k_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.ks[2] + cv * 8) * 2);
     v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
   }
-  auto load_tile = [&](int k0) {
-    const buffer_rsrc kb = make_buffer(kbase + static_cast<int64_t>(k0) * a.ks[2], span_bytes(a.Sk - k0, a.ks[2], D));
-    const buffer_rsrc vb = make_buffer(vbase + static_cast<int64_t>(k0) * a.vs[2], span_bytes(a.Sk - k0, a.vs[2], D));
+  // a cursor walks the key tiles in order: stepping it is four scalar adds instead of 64-bit multiplies
+  const char* k_ptr = reinterpret_cast<const char*>(kbase);
+  const char* v_ptr = reinterpret_cast<const char*>(vbase);
+  uint32_t k_left = span_bytes(a.Sk, a.ks[2], D), v_left = span_bytes(a.Sk, a.vs[2], D);
+  const uint32_t k_step = static_cast<uint32_t>(KT * a.ks[2] * 2), v_step = static_cast<uint32_t>(KT * a.vs[2] * 2);
+  auto load_tile = [&]() {  // the next tile of KT keys
+    const buffer_rsrc kb = make_buffer(k_ptr, k_left), vb = make_buffer(v_ptr, v_left);
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       kreg[i] = buffer_load_b128(kb, k_off[i]);
       vreg[i] = buffer_load_b128(vb, v_off[i]);
     }
+    k_ptr += k_step;  k_left -= k_step;
+    v_ptr += v_step;  v_left -= v_step;
   };
   auto store_tile = [&](int buf) {
     __bf16* sK = smem + buf * C::kTileElems;
@@ -159,7 +166,7 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   };
 
   if (ntiles > 0) {
-    load_tile(0);
+    load_tile();
     store_tile(0);
   }
   // Every load issued so far (Q fragments, the merge state, tile 0) is complete on each path that enters the
@@ -167,14 +174,14 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   // fill.  Saying so here keeps the compiler from putting a vmcnt(0) wait in front of the loop's first MFMAs,
   // where it would wait for the prefetch of the NEXT tile on every trip.
   __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
-  if (ntiles > 1) load_tile(KT);
+  if (ntiles > 1) load_tile();
   __syncthreads();
 
   for (int t = 0; t < ntiles; ++t) {
     // stage tile t+1 into the other buffer (its readers finished before the barrier that ended trip t-1)
     if (t + 1 < ntiles) {
       store_tile((t + 1) & 1);
-      if (t + 2 < ntiles) load_tile((t + 2) * KT);
+      if (t + 2 < ntiles) load_tile();
     }
     const __bf16* sK = smem + (t & 1) * C::kTileElems;
     const __bf16* sV = sK + KT * LDK;
@@ -266,7 +273,8 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     __syncthreads();  // all waves are done with buffer t&1 (it is refilled in trip t+1) and tile t+1 is visible
   }
 
-  // ---- epilogue
+  // ---- epilogue: lse per query; the wave's 32 output rows leave through its piece of LDS as whole lines
+  //      (the loop ended on a barrier, so the tile buffers are free)
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const float l_tot = half_sum(l_run[qb]);
@@ -274,25 +282,18 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     if (live && h == 0)
       p.lse[lse_row0 + qrow[qb]] = l_tot > 0.f ? (m_run[qb] + fast_log2(l_tot)) * kLn2 : -INFINITY;
-    if (!live) continue;
-    const int64_t off = b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(qrow[qb]) * a.os[2];
+    // normalise in place: 1 / l differs per lane (row), the store helper applies one scale to all
 #pragma unroll
     for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int d = 32 * db + 8 * j + 4 * h;
-        if (p.out_f32) {
-          f32x4 v4;
-#pragma unroll
-          for (int t = 0; t < 4; ++t) v4[t] = o[qb][db][4 * j + t] * inv;
-          *reinterpret_cast<f32x4*>(static_cast<float*>(p.out) + off + d) = v4;
-        } else {
-          u32x2 v2;
-          v2[0] = pack_bf16x2(o[qb][db][4 * j] * inv, o[qb][db][4 * j + 1] * inv);
-          v2[1] = pack_bf16x2(o[qb][db][4 * j + 2] * inv, o[qb][db][4 * j + 3] * inv);
-          *reinterpret_cast<u32x2*>(static_cast<__bf16*>(p.out) + off + d) = v2;
-        }
-      }
+      for (int i = 0; i < 16; ++i) o[qb][db][i] *= inv;
+    unsigned char* region = smem_raw + (wave * QB + qb) * kRowRegionBytes;
+    const int row0 = q0 + (wave * QB + qb) * 32;
+    const int64_t off = b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(row0) * a.os[2];
+    if (p.out_f32)
+      wave_store_rows<D, true>(region, o[qb], 1.f, static_cast<float*>(p.out) + off, a.os[2], a.Sq - row0, lane, false, false);
+    else
+      wave_store_rows<D, false>(region, o[qb], 1.f, static_cast<__bf16*>(p.out) + off, a.os[2], a.Sq - row0, lane, false, false);
   }
 }
 
