@@ -50,6 +50,7 @@ struct KvCfg {
   static constexpr size_t kBufBytes = kBufElems * sizeof(__bf16) + 2 * BM * sizeof(float);
   static constexpr size_t kLdsBytes = 2 * kBufBytes;                   // double-buffered
   static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
+  static_assert(NW * WaveTile<D>::kRegionBytes <= kBufBytes, "the K / V fragments pass through the second tile buffer");
 };
 
 template <int D>
@@ -72,21 +73,18 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
   const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
   const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
 
-  // ---- K, V fragments of this wave's 32 keys (B operand: lane = key, 8 consecutive d per k step)
+  // ---- K, V fragments of this wave's 32 keys (B operand: lane = key, 8 consecutive d per k step), fetched
+  //      row-major and turned into fragments through the wave's piece of the SECOND tile buffer, which nothing
+  //      else writes before the end of the first trip, a barrier later
   bf16x8 kf[D / 16], vf[D / 16];
   {
-    const int key = key0 + 32 * wave + n;
-    const bool live = key < a.Sk;
-#pragma unroll
-    for (int s = 0; s < D / 16; ++s) {
-      u32x4 rk = {0, 0, 0, 0}, rv = {0, 0, 0, 0};
-      if (live) {
-        rk = *reinterpret_cast<const u32x4*>(kbase + static_cast<int64_t>(key) * a.ks[2] + 16 * s + 8 * h);
-        rv = *reinterpret_cast<const u32x4*>(vbase + static_cast<int64_t>(key) * a.vs[2] + 16 * s + 8 * h);
-      }
-      kf[s] = __builtin_bit_cast(bf16x8, rk);
-      vf[s] = __builtin_bit_cast(bf16x8, rv);
-    }
+    const int row0 = key0 + 32 * wave;
+    WaveTile<D> kt, vt;
+    kt.issue(make_buffer(kbase + static_cast<int64_t>(row0) * a.ks[2], span_bytes(a.Sk - row0, a.ks[2], D)), a.ks[2], lane);
+    vt.issue(make_buffer(vbase + static_cast<int64_t>(row0) * a.vs[2], span_bytes(a.Sk - row0, a.vs[2], D)), a.vs[2], lane);
+    unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
+    kt.fragments(region, lane, kf);
+    vt.fragments(region, lane, vf);
   }
 
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
@@ -318,6 +316,7 @@ struct DqCfg {
   static constexpr int kTileElems = 2 * KT * LDK;
   static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);  // double-buffered
   static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
+  static_assert(NW * WaveTile<D>::kRegionBytes <= kLdsBytes, "the Q / dO fragments pass through the tile buffers");
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
@@ -342,31 +341,28 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
   const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
   const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
 
-  // ---- per-lane query: Q and dO fragments (B operands), lse and delta
+  // ---- per-lane query: Q and dO fragments (B operands: fetched row-major, turned into fragments through the
+  //      wave's piece of LDS; the tile buffers are filled only after the barrier below), lse and delta
   const int qrow = q0 + wave * 32 + n;
   const bool qlive = qrow < a.Sq;
   bf16x8 qf[D / 16], dof[D / 16];
   float lse2 = INFINITY, delta = 0.f;
   {
-    const int64_t rq = qlive ? qrow : 0;
-    const __bf16* qsrc = a.q + b * a.qs[0] + hq * a.qs[1] + rq * a.qs[2] + 8 * h;
-    const __bf16* dsrc = p.dout + b * a.os[0] + hq * a.os[1] + rq * a.os[2] + 8 * h;
-#pragma unroll
-    for (int s = 0; s < D / 16; ++s) {
-      u32x4 rq4 = {0, 0, 0, 0}, rd4 = {0, 0, 0, 0};
-      if (qlive) {
-        rq4 = *reinterpret_cast<const u32x4*>(qsrc + 16 * s);
-        rd4 = *reinterpret_cast<const u32x4*>(dsrc + 16 * s);
-      }
-      qf[s] = __builtin_bit_cast(bf16x8, rq4);
-      dof[s] = __builtin_bit_cast(bf16x8, rd4);
-    }
+    const int row0 = q0 + wave * 32;
+    WaveTile<D> qt, dt;
+    qt.issue(make_buffer(a.q + b * a.qs[0] + hq * a.qs[1] + static_cast<int64_t>(row0) * a.qs[2],
+                         span_bytes(a.Sq - row0, a.qs[2], D)), a.qs[2], lane);
+    dt.issue(make_buffer(p.dout + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(row0) * a.os[2],
+                         span_bytes(a.Sq - row0, a.os[2], D)), a.os[2], lane);
     if (qlive) {
       const int64_t gi = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + qrow;
       const float l = p.lse[gi];
       lse2 = (l == -INFINITY) ? INFINITY : l * kLog2e;  // a row that saw no key contributes nothing
       delta = p.delta[gi];
     }
+    unsigned char* region = smem_raw + wave * WaveTile<D>::kRegionBytes;
+    qt.fragments(region, lane, qf);
+    dt.fragments(region, lane, dof);
   }
 
   f32x16 dq[D / 32];
@@ -423,10 +419,9 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     }
   };
 
-  if (ntiles > 0) {
-    load_tile();
-    store_tile(0);
-  }
+  if (ntiles > 0) load_tile();
+  __syncthreads();  // every wave has its Q / dO fragments: the tile buffers may be filled
+  if (ntiles > 0) store_tile(0);
   // all loads so far are complete on every path into the loop (the LDS fill waited for the newest); stating
   // it keeps a vmcnt(0) wait, which would hit the next tile's prefetch, out of the loop body
   __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);

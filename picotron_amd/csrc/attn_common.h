@@ -84,6 +84,37 @@ __device__ __forceinline__ float half_sum(float v) {
   return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 
+// ---- reading a wave's 32 x D operand tile as MFMA fragments.  Fetched straight in fragment layout (lane =
+// row, 16 bytes per lane) one instruction touches 32 different lines; fetched row-major -- 16 bytes per lane,
+// 8 or 16 consecutive lanes per row -- the same bytes arrive in a quarter of the line requests, and a detour
+// through a 32 x (D + 8) piece of LDS private to the wave turns them into fragments: lane n gets row n % 32,
+// and for k step s the elements 16s + 8h ..+7 (h = lane / 32).  Rows past the end of the window read as zeros.
+template <int D>
+struct WaveTile {
+  static constexpr int kChunks = D / 16;                 // 16-byte pieces per lane
+  static constexpr int kRegionBytes = 32 * (D + 8) * 2;
+  u32x4 raw[kChunks];
+  __device__ __forceinline__ void issue(buffer_rsrc window, int64_t row_stride, int lane) {
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+      const int idx = lane + 64 * i, r = idx / (D / 8), cv = idx % (D / 8);
+      raw[i] = buffer_load_b128(window, static_cast<uint32_t>((static_cast<int64_t>(r) * row_stride + cv * 8) * 2));
+    }
+  }
+  __device__ __forceinline__ void fragments(unsigned char* region, int lane, bf16x8 (&frag)[D / 16]) const {
+    constexpr int kPitch = (D + 8) * 2;
+#pragma unroll
+    for (int i = 0; i < kChunks; ++i) {
+      const int idx = lane + 64 * i, r = idx / (D / 8), cv = idx % (D / 8);
+      *reinterpret_cast<u32x4*>(region + r * kPitch + cv * 16) = raw[i];
+    }
+    const int n = lane % 32, h = lane / 32;
+#pragma unroll
+    for (int s = 0; s < D / 16; ++s)
+      frag[s] = *reinterpret_cast<const bf16x8*>(region + n * kPitch + (16 * s + 8 * h) * 2);
+  }
+};
+
 // ---- writing a wave's 32 result rows.  The accumulators of the transposed products hold, per lane, one row
 // (lane % 32) and, in registers 4j..4j+3 of block db, columns 32db + 8j + 4h ..+3 (h = lane / 32).  Stored
 // straight from that layout a wave would touch 32 different 128-byte lines with 8 or 16 bytes each per

@@ -35,6 +35,7 @@ struct FwdCfg {
   static constexpr int kTileElems = KT * (LDK + LDV);
   static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);
   static_assert(NW * QB * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
+  static_assert(NW * QB * WaveTile<D>::kRegionBytes <= kLdsBytes, "the Q fragments pass through the tile buffers");
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
@@ -66,20 +67,18 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
   const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
 
-  // ---- Q fragments (B operand of S^T): lane = query, 8 consecutive d per 16-wide k step
+  // ---- Q fragments (B operand of S^T): lane = query, 8 consecutive d per 16-wide k step; fetched row-major and
+  //      turned into fragments through the wave's piece of LDS (the tile buffers are filled only after the
+  //      barrier below)
   bf16x8 qf[QB][D / 16];
   int qrow[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    qrow[qb] = q0 + (wave * QB + qb) * 32 + n;
-    const bool live = qrow[qb] < a.Sq;
-    const __bf16* src = qbase + static_cast<int64_t>(live ? qrow[qb] : 0) * a.qs[2] + 8 * h;
-#pragma unroll
-    for (int s = 0; s < D / 16; ++s) {
-      u32x4 raw = {0, 0, 0, 0};
-      if (live) raw = *reinterpret_cast<const u32x4*>(src + 16 * s);
-      qf[qb][s] = __builtin_bit_cast(bf16x8, raw);
-    }
+    const int row0 = q0 + (wave * QB + qb) * 32;
+    qrow[qb] = row0 + n;
+    WaveTile<D> qt;
+    qt.issue(make_buffer(qbase + static_cast<int64_t>(row0) * a.qs[2], span_bytes(a.Sq - row0, a.qs[2], D)), a.qs[2], lane);
+    qt.fragments(smem_raw + (wave * QB + qb) * WaveTile<D>::kRegionBytes, lane, qf[qb]);
   }
 
   // ---- running state: m in the log2 domain (scores scaled by sm_scale*log2e), l split over the halves
@@ -165,10 +164,9 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     }
   };
 
-  if (ntiles > 0) {
-    load_tile();
-    store_tile(0);
-  }
+  if (ntiles > 0) load_tile();
+  __syncthreads();  // every wave has its Q fragments: the tile buffers may be filled
+  if (ntiles > 0) store_tile(0);
   // Every load issued so far (Q fragments, the merge state, tile 0) is complete on each path that enters the
   // loop, because the LDS fill waited for the newest of them -- but not on the static path that skips the
   // fill.  Saying so here keeps the compiler from putting a vmcnt(0) wait in front of the loop's first MFMAs,
