@@ -65,6 +65,7 @@ class RingBench:
         self.torch, self.ops = torch, ops
         self.B, self.H, self.S, self.D, self.W = B, H, S, D, W
         self.Sc = S // W
+        self.side = torch.cuda.Stream()
         self.scale = 1.0 / math.sqrt(D)
         g = torch.Generator().manual_seed(0)
         q = torch.randn(B, H, S, D, generator=g) * self.scale   # "scaled by 1/sqrt(D) on q"
@@ -132,8 +133,9 @@ class RingBench:
         self.ops.attn_fwd(self.q, self.k, self.v, self.scale, True, 0, out=self.out, lse=self.lse_b)
 
     def backward_kernel_batched(self):
+        # the dQ kernel goes to a second stream: it and the dK/dV kernel are independent
         self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, self.dq_b,
-                          self.dk_b, self.dv_b)
+                          self.dk_b, self.dv_b, side_stream=self.side)
 
     def backward_dkdv_only(self):
         self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, None,

@@ -245,12 +245,14 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
              dq: Optional[torch.Tensor] = None, dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None,
              dq_accumulate: bool = False, dkv_accumulate: bool = False, dq_dtype=torch.float32,
              dkv_dtype=torch.float32, dq_like: Optional[torch.Tensor] = None, want_dq: bool = True,
-             want_dkv: bool = True):
+             want_dkv: bool = True, side_stream: Optional["torch.cuda.Stream"] = None):
     """Gradients of one attention block; returns (dq [B,Hq,Sq,D], dk, dv [B,Hkv,Sk,D]).
 
     Buffers that are passed in are written in place (fp32 ones can be accumulated into: the running dq of a
     rank and the travelling dk / dv of the ring); missing ones are allocated in the requested dtype, dq with
     the strides of `dq_like` if given.  want_dq / want_dkv = False skips that gradient (and its kernel).
+    With `side_stream` the dQ kernel is enqueued there and the dK/dV kernel on the current stream (the two are
+    independent; each one's ramp-up and tail overlap the other); the current stream waits for both.
     """
     _dev(dout, q, k, v, lse, delta, dq, dk, dv)
     q, k, v, dout = _attn_in(q, "q"), _attn_in(k, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
@@ -281,10 +283,23 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
     d = _desc(q, k, v, dout, sm_scale, causal, q_offset)
     dqs = (ctypes.c_int64 * 3)(*(dq.stride()[:3] if dq is not None else (0, 0, 0)))
     dks = (ctypes.c_int64 * 3)(*(dk.stride()[:3] if dk is not None else (0, 0, 0)))
-    check(_lib.lib().pico_attn_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(lse.contiguous()),
-                                   _ptr(delta.contiguous()), _ptr(dq), dqs, _dt(dq, "dq") if dq is not None else PICO_F32,
-                                   int(dq_accumulate), _ptr(dk), _ptr(dv), dks,
-                                   _dt(dk, "dk/dv") if dk is not None else PICO_F32, int(dkv_accumulate), _stream()))
+    lse_c, delta_c = lse.contiguous(), delta.contiguous()
+
+    def launch(dq_, dk_, dv_):
+        check(_lib.lib().pico_attn_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(lse_c), _ptr(delta_c),
+                                       _ptr(dq_), dqs, _dt(dq, "dq") if dq is not None else PICO_F32, int(dq_accumulate),
+                                       _ptr(dk_), _ptr(dv_), dks, _dt(dk, "dk/dv") if dk is not None else PICO_F32,
+                                       int(dkv_accumulate), _stream()))
+
+    if side_stream is not None and dq is not None and dk is not None:
+        cur = torch.cuda.current_stream()
+        side_stream.wait_stream(cur)
+        with torch.cuda.stream(side_stream):
+            launch(dq, None, None)
+        launch(None, dk, dv)
+        cur.wait_stream(side_stream)
+    else:
+        launch(dq, dk, dv)
     return dq, dk, dv
 
 

@@ -52,6 +52,13 @@ def test_argument_checks_run_without_a_gpu():
     assert lib.pico_attn_fwd(ctypes.byref(d), None, None, None, None, None, 0, 0, None) == -3   # head_dim
     assert b"head_dim" in lib.pico_last_error()
     assert lib.pico_rmsnorm_bwd_workspace_bytes(4096, 2048) == 512 * 2048 * 4
+    # the kernels address one head's rows through 32-bit byte offsets: a 4 GiB span is refused
+    d.D, d.Sq, d.Sk = 64, 64, 64
+    for st in (d.q_stride, d.k_stride, d.v_stride, d.o_stride):
+        st[0], st[1], st[2] = 64 * 64 * 3, 64 * 64, 64
+    d.k_stride[2] = 1 << 26
+    assert lib.pico_attn_fwd(ctypes.byref(d), None, None, None, None, None, 0, 0, None) == -5
+    assert b"4 GiB" in lib.pico_last_error()
 
 
 def test_cpu_tensors_are_refused_not_computed():

@@ -326,6 +326,36 @@ def test_attn_bwd_bf16_strided_outputs_and_determinism(ops, device):
         assert rel_l2(x, y) <= 5e-3
 
 
+def test_attn_bwd_side_stream_matches_one_stream(ops, device):
+    """The dQ kernel on a second stream changes scheduling only: bit-identical gradients."""
+    B, H, S, D = 2, 4, 320, 64
+    q, k, v = (t.to(device) for t in attn_inputs(B, H, H, S, S, D, seed=86))
+    do = rnd(B, H, S, D, seed=87).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(q, k, v, 0.125, True)
+    delta = ops.attn_bwd_preprocess(do, out)
+    one = ops.attn_bwd(do, q, k, v, lse, delta, 0.125, True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16)
+    side = torch.cuda.Stream()
+    for _ in range(3):
+        two = ops.attn_bwd(do, q, k, v, lse, delta, 0.125, True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16,
+                           side_stream=side)
+        torch.cuda.synchronize()
+        for x, y in zip(one, two):
+            assert torch.equal(x, y)
+
+
+def test_attn_rejects_unsupported_layouts(ops, device):
+    """Error behaviour of the boundary: gradient rows that are not 16-byte aligned raise, nothing is launched."""
+    B, H, S, D = 1, 2, 64, 64
+    q, k, v = (t.to(device) for t in attn_inputs(B, H, H, S, S, D, seed=88))
+    do = rnd(B, H, S, D, seed=89).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(q, k, v, 0.125, True)
+    delta = ops.attn_bwd_preprocess(do, out)
+    # dk / dv rows 68 elements apart: not a multiple of 8
+    pad = torch.empty(B, H, S, D + 4, dtype=torch.bfloat16, device=device)
+    with pytest.raises(RuntimeError, match="strides"):
+        ops.attn_bwd(do, q, k, v, lse, delta, 0.125, True, 0, None, pad[..., :D], pad.clone()[..., :D], want_dq=False)
+
+
 def test_attn_empty_inputs(ops, device):
     """No queries or no keys: nothing faults; gradients of the side that exists are zero."""
     z = torch.zeros(1, 2, 0, 64, dtype=torch.bfloat16, device=device)
