@@ -41,7 +41,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one dK/dV launch at the bench shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy
 # kernel of known size (see profiles/); None until measured
-TRAFFIC_BYTES_DKDV = 123.3e6
+TRAFFIC_BYTES_DKDV = 103.8e6
 
 
 def parse():
@@ -65,7 +65,6 @@ class RingBench:
         self.torch, self.ops = torch, ops
         self.B, self.H, self.S, self.D, self.W = B, H, S, D, W
         self.Sc = S // W
-        self.side = torch.cuda.Stream()
         self.scale = 1.0 / math.sqrt(D)
         g = torch.Generator().manual_seed(0)
         q = torch.randn(B, H, S, D, generator=g) * self.scale   # "scaled by 1/sqrt(D) on q"
@@ -133,9 +132,8 @@ class RingBench:
         self.ops.attn_fwd(self.q, self.k, self.v, self.scale, True, 0, out=self.out, lse=self.lse_b)
 
     def backward_kernel_batched(self):
-        # the dQ kernel goes to a second stream: it and the dK/dV kernel are independent
         self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, self.dq_b,
-                          self.dk_b, self.dv_b, side_stream=self.side)
+                          self.dk_b, self.dv_b)
 
     def backward_dkdv_only(self):
         self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, None,
@@ -177,8 +175,10 @@ class RingBench:
         self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
 
 
-def graph_time(torch, fn, iters, warmup=3):
-    """Records fn() once into a HIP graph and returns (ms per replay over `iters` replays, graph)."""
+def graph_time(torch, fn, iters, warmup=3, per_graph=1):
+    """Records fn() `per_graph` times into a HIP graph and returns (ms per fn() over `iters` replays, graph).
+    Each replay is one graph launch, and the GPU idles for about 8 us between two of them; with several
+    calls recorded per graph that gap is shared out, as it is in a training step recorded as one graph."""
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -188,7 +188,8 @@ def graph_time(torch, fn, iters, warmup=3):
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        fn()
+        for _ in range(per_graph):
+            fn()
     for _ in range(2):
         graph.replay()
     torch.cuda.synchronize()
@@ -198,7 +199,7 @@ def graph_time(torch, fn, iters, warmup=3):
         graph.replay()
     stop.record()
     torch.cuda.synchronize()
-    return start.elapsed_time(stop) / iters, graph
+    return start.elapsed_time(stop) / (iters * per_graph), graph
 
 
 def bandwidth_extras(torch, ops, iters=50):
@@ -399,13 +400,17 @@ def main():
         rb.step_batched()
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
+    # several steps are recorded per graph (the largest divisor of K up to 20) so that exactly K steps are timed and
+    # the idle time between two graph launches is not charged to every single step
+    per_graph = max(g for g in range(1, 21) if args.steps % g == 0)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        rb.step_batched()
+        for _ in range(per_graph):
+            rb.step_batched()
     graph.replay()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for _ in range(args.steps // per_graph):
         graph.replay()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
@@ -415,7 +420,7 @@ def main():
     # ---- dominant kernel: the dK/dV launch alone, HIP events on the launching stream.  Its algorithmic work
     #      is 4 of the backward's 5 matrix products (S, dP, dV, dK): 8 FLOPs per (query, key, d) triple.
     dkdv_flops = bwd_flops * 0.8
-    ms_dkdv, _ = graph_time(torch, rb.backward_dkdv_only, max(args.steps // 2, 10))
+    ms_dkdv, _ = graph_time(torch, rb.backward_dkdv_only, max(args.steps // 10, 10), per_graph=10)
     dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel_d64", "achieved": round(dkdv_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
@@ -423,14 +428,14 @@ def main():
 
     extras = {}
     if not args.no_extras:
-        ms_dq, _ = graph_time(torch, rb.backward_dq_only, max(args.steps // 2, 10))
-        ms_bwd_k, _ = graph_time(torch, rb.backward_kernel_batched, max(args.steps // 2, 10))
+        ms_dq, _ = graph_time(torch, rb.backward_dq_only, max(args.steps // 10, 10), per_graph=10)
+        ms_bwd_k, _ = graph_time(torch, rb.backward_kernel_batched, max(args.steps // 10, 10), per_graph=10)
         extras["attn_bwd_dq_kernel"] = {"us_per_launch": round(ms_dq * 1e3, 2),
                                         "TFLOP/s_algorithmic": round(bwd_flops * 0.2 / (ms_dq * 1e-3) / 1e12, 2),
                                         "TFLOP/s_executed": round(bwd_flops * 0.6 / (ms_dq * 1e-3) / 1e12, 2),
                                         "note": "recomputes S and dP: executes 3 products for 1 algorithmic"}
         extras["attn_bwd_both_kernels"] = {"us": round(ms_bwd_k * 1e3, 2), "TFLOP/s_algorithmic": round(bwd_flops / (ms_bwd_k * 1e-3) / 1e12, 2)}
-        ms_fwd, _ = graph_time(torch, rb.forward_batched, max(args.steps // 2, 10))
+        ms_fwd, _ = graph_time(torch, rb.forward_batched, max(args.steps // 10, 10), per_graph=10)
         extras["attn_fwd_kernel"] = {"TFLOP/s": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2), "us_per_launch": round(ms_fwd * 1e3, 2),
                                      "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
         ms_rank, _ = graph_time(torch, rb.step, max(args.steps // 4, 10))
@@ -453,7 +458,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: causal ring attention fwd+bwd, B4 H32 S1024 D64, cp_size 4, the ring steps of all "
                                "4 ranks on one GPU (ranks batched into one launch per direction)",
-                   "global_batch": 4, "seq_len": 1024, "flops_per_step": total_flops},
+                   "global_batch": 4, "seq_len": 1024, "flops_per_step": total_flops, "steps_per_graph_launch": per_graph},
         "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": roofline,
     }

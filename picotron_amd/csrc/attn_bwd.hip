@@ -37,6 +37,12 @@ struct BwdParams {
 };
 
 // =====================================================================================  dK / dV
+// bf16 gradients leave with streaming (non-temporal) stores unless built with -DPICO_STREAM_GRADS=0
+#ifndef PICO_STREAM_GRADS
+#define PICO_STREAM_GRADS 1
+#endif
+constexpr bool kStreamGrads = PICO_STREAM_GRADS != 0;
+
 template <int D>
 struct KvCfg {
   static constexpr int NW = 4;
@@ -287,8 +293,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
       wave_store_rows<D, true>(region, dk_acc, a.sm_scale, static_cast<float*>(p.dk) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
       wave_store_rows<D, true>(region, dv_acc, 1.f, static_cast<float*>(p.dv) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
     } else {
-      wave_store_rows<D, false>(region, dk_acc, a.sm_scale, static_cast<__bf16*>(p.dk) + off, p.dks[2], rows_live, lane, false, true);
-      wave_store_rows<D, false>(region, dv_acc, 1.f, static_cast<__bf16*>(p.dv) + off, p.dks[2], rows_live, lane, false, true);
+      wave_store_rows<D, false>(region, dk_acc, a.sm_scale, static_cast<__bf16*>(p.dk) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
+      wave_store_rows<D, false>(region, dv_acc, 1.f, static_cast<__bf16*>(p.dv) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
     }
   }
 }
@@ -504,7 +510,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     if (p.dq_f32)
       wave_store_rows<D, true>(region, dq, a.sm_scale, static_cast<float*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, p.dq_accumulate, false);
     else
-      wave_store_rows<D, false>(region, dq, a.sm_scale, static_cast<__bf16*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, false, true);
+      wave_store_rows<D, false>(region, dq, a.sm_scale, static_cast<__bf16*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, false, kStreamGrads);
   }
 }
 

@@ -69,17 +69,6 @@ class SwiGLUFunc(torch.autograd.Function):
         return ops.swiglu_bwd(dy, gate, up)
 
 
-_SIDE = {}
-
-
-def _side_stream(device):
-    """One extra stream per device for the dQ kernel of the attention backward (default priority)."""
-    key = torch.device(device).index
-    if key not in _SIDE:
-        _SIDE[key] = torch.cuda.Stream(device=device)
-    return _SIDE[key]
-
-
 class FlashAttnFunc(torch.autograd.Function):
     """Single-chunk causal / dense attention on [B,H,S,D] views; K/V may carry fewer (GQA) heads."""
 
@@ -96,5 +85,5 @@ class FlashAttnFunc(torch.autograd.Function):
         delta = ops.attn_bwd_preprocess(dout, out)
         # gradients come back in the dtype and memory layout of their inputs: no accumulation buffer, no cast pass
         dq, dk, dv = ops.attn_bwd(dout, q, k, v, lse, delta, ctx.sm_scale, ctx.causal, 0, dq_dtype=q.dtype, dq_like=q,
-                                  dkv_dtype=k.dtype, side_stream=_side_stream(q.device))
+                                  dkv_dtype=k.dtype)
         return dq, dk, dv, None, None

@@ -252,7 +252,9 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
     rank and the travelling dk / dv of the ring); missing ones are allocated in the requested dtype, dq with
     the strides of `dq_like` if given.  want_dq / want_dkv = False skips that gradient (and its kernel).
     With `side_stream` the dQ kernel is enqueued there and the dK/dV kernel on the current stream (the two are
-    independent; each one's ramp-up and tail overlap the other); the current stream waits for both.
+    independent); the current stream waits for both.  Measured on MI355X it is a wash at the benchmark shape
+    (+3 % on one box, -4 % on another: the fork / join costs what the overlapped tails save), so nothing in
+    this package turns it on by default.
     """
     _dev(dout, q, k, v, lse, delta, dq, dk, dv)
     q, k, v, dout = _attn_in(q, "q"), _attn_in(k, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
