@@ -216,12 +216,19 @@ def bandwidth_extras(torch, ops, iters=50):
             def body():
                 for s_ in sets:
                     call(*s_)
-            ms, _ = graph_time(torch, body, iters)
+            # the warm variant records ten calls per graph so that the idle time between graph launches is shared out
+            ms, _ = graph_time(torch, body, iters, per_graph=10 if nsets == 1 else 1)
             gbs = bytes_per_call * nsets / (ms * 1e-3) / 1e9
             res[f"{name}_{label}"] = {"GB/s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 3),
                                       "us_per_call": round(ms * 1e3 / nsets, 2), "algorithmic_MB": round(bytes_per_call / 1e6, 2)}
             del sets
 
+    # what the memory system gives a plain device-to-device copy of the same sizes (torch's copy kernel): the
+    # practical ceiling for a read-once / write-once kernel at this size, well below the 8 TB/s pin rate
+    run("copy_33MB_reference", lambda: (torch.randn(T, h, device=dev).to(bf), torch.empty(T, h, dtype=bf, device=dev)),
+        lambda x, y: y.copy_(x), 2 * T * h * 2, 24)
+    run("copy_201MB_reference", lambda: (torch.randn(T, 3 * I // 2, device=dev).to(bf), torch.empty(T, 3 * I // 2, dtype=bf, device=dev)),
+        lambda x, y: y.copy_(x), 2 * T * (3 * I // 2) * 2, 4)
     w = torch.ones(h, dtype=bf, device=dev)
     run("rmsnorm_fwd", lambda: (torch.randn(T, h, device=dev).to(bf),),
         lambda x: ops.rmsnorm_fwd(x, w, 1e-5, False), 2 * T * h * 2 + h * 2, 24)

@@ -169,8 +169,9 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
 }
 
 // Row-per-wave backward (hidden <= 64 * NV vectors): a wave keeps the packed x / dy of its row in
-// registers, prefetches the next row while it reduces the current one, and carries its share of
-// dweight in registers across all its rows.  The block's four waves are summed through LDS once at
+// registers and carries its share of dweight in registers across all its rows.  No software prefetch of the
+// next row: loads and stores retire in one order, so waiting for a prefetched row also waits for the stores
+// of the current one (measured: 3.4 TB/s with the prefetch, 5.2 TB/s -- the rate of a plain copy -- without).  The block's four waves are summed through LDS once at
 // the end and the block writes one row of the partial-sum workspace.
 template <typename T, int NV>
 __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
@@ -184,8 +185,8 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
   const int nvec = hidden / V;
   const float inv_h = 1.f / static_cast<float>(hidden);
   float dw[NV][V], wv[NV][V];
-  u32x4 xr[2][NV], dr[2][NV];
-  float rs[2];
+  u32x4 xr[NV], dr[NV];
+  float rs;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
 #pragma unroll
@@ -194,16 +195,15 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
   }
   const int64_t stride = static_cast<int64_t>(gridDim.x) * NWAVE;
   int64_t row = static_cast<int64_t>(blockIdx.x) * NWAVE + wave;
-  auto fetch = [&](int buf, int64_t r) {
-    const int64_t rc = r < rows ? r : rows - 1;  // clamped: the values of a dead row are never used
+  auto fetch = [&](int64_t r) {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int v = t + j * kWave;
       const int vc = v < nvec ? v : 0;
-      xr[buf][j] = *reinterpret_cast<const u32x4*>(x + rc * hidden + vc * V);
-      dr[buf][j] = *reinterpret_cast<const u32x4*>(dy + rc * hidden + vc * V);
+      xr[j] = *reinterpret_cast<const u32x4*>(x + r * hidden + vc * V);
+      dr[j] = *reinterpret_cast<const u32x4*>(dy + r * hidden + vc * V);
     }
-    rs[buf] = rstd[rc];
+    rs = rstd[r];
   };
   auto unpack = [&](const u32x4& raw, float (&out)[V]) {
     if constexpr (V == 8) {
@@ -217,18 +217,16 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
       for (int i = 0; i < 4; ++i) out[i] = __uint_as_float(raw[i]);
     }
   };
-  fetch(0, row);
-  int cur = 0;
-  for (; row < rows; row += stride, cur ^= 1) {
-    fetch(cur ^ 1, row + stride);
-    const float r = rs[cur];
+  for (; row < rows; row += stride) {
+    fetch(row);
+    const float r = rs;
     float c = 0.f;
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       if (t + j * kWave < nvec) {
         float xv[V], dv[V];
-        unpack(xr[cur][j], xv);
-        unpack(dr[cur][j], dv);
+        unpack(xr[j], xv);
+        unpack(dr[j], dv);
 #pragma unroll
         for (int e = 0; e < V; ++e) {
           const float xh = xv[e] * r;
@@ -243,8 +241,8 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
       const int v = t + j * kWave;
       if (v < nvec) {
         float xv[V], dv[V], o[V];
-        unpack(xr[cur][j], xv);
-        unpack(dr[cur][j], dv);
+        unpack(xr[j], xv);
+        unpack(dr[j], dv);
 #pragma unroll
         for (int e = 0; e < V; ++e) o[e] = r * (dv[e] * wv[j][e] - xv[e] * r * c);
         io<T>::store(dx + row * hidden + v * V, o);
