@@ -32,6 +32,7 @@ struct BwdParams {
   void* dv;
   int dq_f32, dq_accumulate;
   int dkv_f32, dkv_accumulate;
+  int pair_ktiles;  // dK/dV kernel: a workgroup takes key tile t and then tile n-1-t (equal work under a causal mask)
   int64_t dqs[3];  // element strides (b, h, s) of dq
   int64_t dks[3];  // element strides (b, h, s) of dk and dv
 };
@@ -60,16 +61,13 @@ struct KvCfg {
 };
 
 template <int D>
-__device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
+__device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int ktile) {
   using C = KvCfg<D>;
   constexpr int BM = C::BM, BN = C::BN, LDQ = C::LDQ;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
   const AttnParams& a = p.a;
-  // grid = (Hkv * B, key tiles): the x index runs fastest in dispatch order, so all heads of key tile 0
-  // (the longest under a causal mask) start first and the short tiles fill in behind them; workgroups of
-  // one head are a multiple of 8 apart in dispatch order and so share an XCD's L2
-  const int ktile = blockIdx.y, hkv = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
+  const int hkv = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
   const int group = a.Hq / a.Hkv;
   const int key0 = ktile * BN;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
@@ -296,6 +294,24 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
       wave_store_rows<D, false>(region, dk_acc, a.sm_scale, static_cast<__bf16*>(p.dk) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
       wave_store_rows<D, false>(region, dv_acc, 1.f, static_cast<__bf16*>(p.dv) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
     }
+  }
+}
+
+// grid = (Hkv * B, key tiles or pairs of key tiles): the x index runs fastest in dispatch order, so all heads of
+// key tile 0 (the longest under a causal mask) start first and the short tiles fill in behind them; workgroups
+// of one head are a multiple of 8 apart in dispatch order and so share an XCD's L2.  With pair_ktiles a
+// workgroup takes tile t and then tile n-1-t: under a causal mask every pair is the same amount of work, so a
+// launch whose pairs fill the GPU once ends without a tail of short workgroups and pays the start-up of a
+// workgroup (kernel arguments, first loads) half as often.
+template <int D>
+__device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
+  const int n_ktiles = (p.a.Sk + KvCfg<D>::BN - 1) / KvCfg<D>::BN;
+  const int first = blockIdx.y;
+  attn_bwd_dkdv_tile<D>(p, first);
+  const int second = n_ktiles - 1 - first;
+  if (p.pair_ktiles && second != first) {
+    __syncthreads();  // the epilogue's pieces of LDS are the next tile's buffers
+    attn_bwd_dkdv_tile<D>(p, second);
   }
 }
 
@@ -574,7 +590,12 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
     attr_set = true;
   }
   const int n_ktiles = (p.a.Sk + C::BN - 1) / C::BN;
-  hipLaunchKernelGGL(KvKernel<D>::fn, dim3(p.a.Hkv * p.a.B, n_ktiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  // pairs only when they still fill the GPU (two workgroups per CU for D = 64, one for D = 128)
+  BwdParams q = p;
+  const int64_t slots = D == 64 ? 512 : 256;
+  q.pair_ktiles = p.a.causal && n_ktiles >= 2 && static_cast<int64_t>(p.a.Hkv) * p.a.B * ((n_ktiles + 1) / 2) >= slots;
+  const int grid_y = q.pair_ktiles ? (n_ktiles + 1) / 2 : n_ktiles;
+  hipLaunchKernelGGL(KvKernel<D>::fn, dim3(p.a.Hkv * p.a.B, grid_y), dim3(C::kThreads), C::kLdsBytes, s, q);
   return PICO_OK;
 }
 
