@@ -51,7 +51,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels")
-    ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B-shaped training step")
+    ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B- and Llama-2-7B-shaped training steps")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: a few launches of a plain copy of known size and of each attention kernel "
                          "at the bench shape, nothing else (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -126,6 +126,15 @@ class RingBench:
     def step(self):
         self.forward()
         self.backward()
+
+    def step_one_rank(self, r):
+        """Forward + backward of cp rank r alone: its query chunk against chunks 0..r (one launch per direction)."""
+        ops = self.ops
+        q, k, v, do, out, dk, dv = self._views(r)
+        ops.attn_fwd(q, k, v, self.scale, True, r * self.Sc, out=out, lse=self.lse[r])
+        delta = ops.attn_bwd_preprocess(do, out, delta=self.delta[r])
+        ops.attn_bwd(do, q, k, v, self.lse[r], delta, self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
+                     dkv_accumulate=True)
 
     # -- all four ranks in one launch per direction (q_offset 0 over the whole sequence)
     def forward_batched(self):
@@ -246,19 +255,21 @@ def bandwidth_extras(torch, ops, iters=50):
     return res
 
 
-def train_step_extra(torch, steps=8, warmup=3):
-    """configs[2]: SmolLM-1.7B-shaped training step (24 layers, h 2048, 32 heads, I 8192, V 49152), mbs 4,
-    seq 1024, bf16 parameters with fp32 AdamW master weights and moments, random init, synthetic tokens."""
+def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
+    """configs[2]: SmolLM-1.7B-shaped training step (24 layers, h 2048, 32 heads of 64, I 8192, V 49152), mbs 4, seq 1024;
+    configs[3]: Llama-2-7B-shaped step (32 layers, h 4096, 32 heads of 128, I 11008, V 32000), mbs 1, seq 4096.
+    bf16 parameters with fp32 AdamW master weights and moments, random init, synthetic tokens."""
     import torch.nn.functional as F
 
     import picotron_amd.process_group_manager as pgm
-    from oracle.model import smollm_1p7b, synthetic_batch
+    from oracle.model import llama2_7b, smollm_1p7b, synthetic_batch
     from picotron_amd.model import Llama
     from picotron_amd.utils import MI355X_BF16_DENSE_FLOPS, flops_per_token, get_num_params
 
     pgm.setup_process_group_manager(1, 1, 1, 1)
     os.environ["CONTEXT_PARALLEL"] = "0"
-    cfg = smollm_1p7b(1024)
+    mbs, seq = (4, 1024) if which == "smollm_1p7b" else (1, 4096)
+    cfg = smollm_1p7b(seq) if which == "smollm_1p7b" else llama2_7b(seq)
     torch.manual_seed(42)
     with torch.device("cuda"):
         model = Llama(cfg)
@@ -268,14 +279,14 @@ def train_step_extra(torch, steps=8, warmup=3):
     for m in master:
         m.grad = torch.zeros_like(m)
     opt = torch.optim.AdamW(master, lr=3e-4, fused=True)
-    ids, tgt = synthetic_batch(cfg.vocab_size, 4, 1024, seed=0)
+    ids, tgt = synthetic_batch(cfg.vocab_size, mbs, seq, seed=0)
     ids, tgt = ids.cuda(), tgt.cuda()
 
     def step():
         for p in params:
             p.grad = None
         logits = model(input_ids=ids)
-        loss = F.cross_entropy(logits.view(4 * 1024, -1).float(), tgt.reshape(-1), reduction="mean")
+        loss = F.cross_entropy(logits.view(mbs * seq, -1).float(), tgt.reshape(-1), reduction="mean")
         loss.backward()
         with torch.no_grad():
             torch._foreach_copy_([m.grad for m in master], [p.grad for p in params])
@@ -293,8 +304,8 @@ def train_step_extra(torch, steps=8, warmup=3):
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
     n = get_num_params(model)
-    tok_s = 4 * 1024 / dt
-    fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, 1024)
+    tok_s = mbs * seq / dt
+    fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, seq)
     res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
            "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
            "note": "attention / RMSNorm / RoPE / SwiGLU on the HIP kernels; projections, CE and AdamW on torch"}
@@ -366,6 +377,24 @@ def cpu_baseline(host_tensors, W, scale, flops_total):
         out[label] = {"value": round(flops_total / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "s_per_step": round(dt, 3)}
     torch.set_num_threads(cores)
     return out
+
+
+def cpu_configs0_step(threads):
+    """configs[0], the reference's own CPU-runnable case, on the CPU oracle: SmolLM-135M-shaped model cut to 2 layers,
+    fp32, B 2, S 256, one full training step (forward, CE, backward, AdamW); seconds per step after one warm-up step."""
+    import torch
+    from oracle.model import OracleLlama, smollm_135m_2layer, synthetic_batch, train_step
+    torch.set_num_threads(threads)
+    torch.manual_seed(42)
+    cfg = smollm_135m_2layer(256)
+    model = OracleLlama(cfg)
+    opt = torch.optim.AdamW(model.parameters(), lr=3e-4)
+    ids, tgt = synthetic_batch(cfg.vocab_size, 2, 256, seed=0)
+    train_step(model, opt, ids, tgt)
+    t0 = time.perf_counter()
+    for _ in range(2):
+        train_step(model, opt, ids, tgt)
+    return (time.perf_counter() - t0) / 2
 
 
 def main():
@@ -447,6 +476,10 @@ def main():
                                      "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
         ms_rank, _ = graph_time(torch, rb.step, max(args.steps // 4, 10))
         extras["one_launch_per_rank"] = {"TFLOP/s": round(total_flops / (ms_rank * 1e-3) / 1e12, 2), "ms_per_step": round(ms_rank, 4)}
+        ms_r3, _ = graph_time(torch, lambda: rb.step_one_rank(3), max(args.steps // 10, 10), per_graph=10)
+        r3_flops = total_flops * 3.5 / 8.0   # 1 causal + 3 dense chunk-blocks of the 8 block-equivalents of all ranks
+        extras["rank3_of_4_alone"] = {"TFLOP/s": round(r3_flops / (ms_r3 * 1e-3) / 1e12, 2), "us_per_step": round(ms_r3 * 1e3, 2),
+                                      "flops": r3_flops}
         ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
         extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4)}
         t0 = time.perf_counter()
@@ -457,7 +490,8 @@ def main():
         extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
         extras["configs4_long_context_rank7_of_8"] = long_context_extra(torch, ops)
         if not args.no_train:
-            extras["smollm_1p7b_train_step"] = train_step_extra(torch)
+            extras["smollm_1p7b_train_step"] = train_step_extra(torch, "smollm_1p7b")
+            extras["llama2_7b_train_step"] = train_step_extra(torch, "llama2_7b", steps=4, warmup=2)
 
     line = {
         "metric": "causal ring-attn fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s",
@@ -475,6 +509,10 @@ def main():
         line["cpu_baseline"] = {"value": main_leg["value"], "unit": "TFLOP/s", "cores": main_leg["cores"], "kind": "port",
                                 "sample": f"full configs[1] shape (fwd+bwd of all 4 ranks), fp32, {main_leg['s_per_step']} s per step; "
                                           f"one thread: {cpu['one_thread']['value']} TFLOP/s ({cpu['one_thread']['s_per_step']} s per step)"}
+        c0_all, c0_one = cpu_configs0_step(main_leg["cores"]), cpu_configs0_step(1)
+        line["cpu_baseline"]["configs0_step"] = {"tokens_per_s_all_threads": round(512 / c0_all, 1), "s_per_step_all_threads": round(c0_all, 3),
+                                                 "tokens_per_s_one_thread": round(512 / c0_one, 1), "s_per_step_one_thread": round(c0_one, 3),
+                                                 "what": "configs[0]: 2-layer SmolLM-135M shape, fp32, B2 S256, full training step on the CPU oracle"}
     if extras:
         line["extras"] = extras
     print(json.dumps(line))
