@@ -17,6 +17,7 @@ struct FwdParams {
   float* lse;
   int out_f32;
   int merge;
+  int pair_order;  // dispatch order of the query tiles, see the kernel
 };
 
 template <int D, int QB, int NW, int KT>
@@ -55,8 +56,11 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   const AttnParams& a = p.a;
   const int n_qtiles = (a.Sq + BM - 1) / BM;
   // grid = (Hq * B, query tiles): x runs fastest in dispatch order, so every head's last query tile (the
-  // longest under a causal mask) starts first and the short tiles fill in behind
-  const int qtile = n_qtiles - 1 - static_cast<int>(blockIdx.y);
+  // longest under a causal mask) starts first and the short tiles fill in behind.  When the whole launch is
+  // resident at once (pair_order), workgroups j and j + (half the grid) share a CU, so the second half runs
+  // the short tiles in ASCENDING order: every CU then holds a long and a short tile of equal total length.
+  const int y = static_cast<int>(blockIdx.y), half = (n_qtiles + 1) / 2;
+  const int qtile = (p.pair_order && y >= half) ? y - half : n_qtiles - 1 - y;
   const int hq = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
   const int hkv = hq / (a.Hq / a.Hkv);
   const int q0 = qtile * BM;
@@ -306,7 +310,9 @@ int launch(const FwdParams& p, hipStream_t s) {
     attr_set = true;
   }
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
-  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW, KT>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  FwdParams q = p;
+  q.pair_order = p.a.causal && n_qtiles >= 2 && static_cast<int64_t>(p.a.Hq) * p.a.B * n_qtiles <= 512;
+  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW, KT>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, q);
   return PICO_OK;
 }
 
