@@ -343,6 +343,28 @@ def test_attn_bwd_side_stream_matches_one_stream(ops, device):
             assert torch.equal(x, y)
 
 
+def test_attn_bwd_paired_key_tiles_match_unpaired(ops, device):
+    """A big causal launch lets each dK/dV workgroup take key tiles t and n-1-t; a launch of half the batch is too
+    small for that and takes one tile per workgroup.  Same arithmetic per head, so the results are bit-identical --
+    with an odd number of key tiles (the middle one has no partner) and a ragged last tile."""
+    B, H, S, D = 8, 16, 1100, 64
+    q, k, v = (t.to(device) for t in attn_inputs(B, H, H, S, S, D, seed=90))
+    do = rnd(B, H, S, D, seed=91).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(q, k, v, 0.125, True)
+    delta = ops.attn_bwd_preprocess(do, out)
+    whole = ops.attn_bwd(do, q, k, v, lse, delta, 0.125, True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16)
+    for half in (slice(0, 4), slice(4, 8)):
+        part = ops.attn_bwd(do[half], q[half], k[half], v[half], lse[half].contiguous(), delta[half].contiguous(), 0.125,
+                            True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16)
+        for x, y in zip(whole, part):
+            assert torch.equal(x[half], y)
+    # and against the oracle on one head of it
+    qf, kf, vf = (t[:1, :1].float().cpu().requires_grad_() for t in (q, k, v))
+    w_o, _ = OR.full_attention_closed_form(qf, kf, vf, 0.125, True, 0)
+    gq, gk, gv = torch.autograd.grad(w_o, (qf, kf, vf), do[:1, :1].float().cpu())
+    assert rel_l2(whole[1][:1, :1], gk) <= 1e-2 and rel_l2(whole[2][:1, :1], gv) <= 1e-2 and rel_l2(whole[0][:1, :1], gq) <= 1e-2
+
+
 def test_attn_rejects_unsupported_layouts(ops, device):
     """Error behaviour of the boundary: gradient rows that are not 16-byte aligned raise, nothing is launched."""
     B, H, S, D = 1, 2, 64, 64
