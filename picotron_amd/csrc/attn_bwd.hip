@@ -43,6 +43,10 @@ struct BwdParams {
 #define PICO_STREAM_GRADS 1
 #endif
 constexpr bool kStreamGrads = PICO_STREAM_GRADS != 0;
+#ifndef PICO_PIPELINE_TRIP
+#define PICO_PIPELINE_TRIP 1
+#endif
+constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 
 template <int D>
 struct KvCfg {
@@ -203,23 +207,17 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     // tile it+1 travels global -> registers while this trip computes; it goes to the other LDS buffer at
     // the end of the trip (that buffer's readers finished before the barrier that ended trip it-1)
     const bool has_next = it + 1 < n_iter;
-    if (has_next) {
-      advance();
-      prefetch();
-    }
+    if (has_next) advance();
     const int q0 = tile * BM;
     const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + buf_off);
     const __bf16* sdO = sQ + BM * LDQ;
     const float* sL = reinterpret_cast<const float*>(sdO + BM * LDQ);
     const float* sDelta = sL + BM;
 
-#pragma unroll
-    for (int sb = 0; sb < BM / 32; ++sb) {
-      const int qs_pos = a.q_offset + q0 + 32 * sb;       // position of the sub-block's first query
-      if (a.causal && kw0 > qs_pos + 31) continue;        // every (query, key) pair of this block is masked
-      // the dP accumulator starts at -delta of its row (sDelta holds the negated value), so dP - delta
-      // comes out of the MFMA
-      f32x16 s_acc, dp_acc;
+    // The three phases of a 32-query sub-block.
+    // products(): S = Q K^T and dP = dO V^T (C tile: lane = key, registers = queries); the dP accumulator starts at
+    // -delta of its row (sDelta holds the negated value), so dP - delta comes out of the MFMA.
+    auto products = [&](int sb, f32x16& s_acc, f32x16& dp_acc) {
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
@@ -233,28 +231,32 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
         s_acc = mfma32(qa, kf[s], s_acc);
         dp_acc = mfma32(da, vf[s], dp_acc);
       }
-      // P = exp2(S*c - lse*log2e), dS = P * (dP - delta) [already in the accumulator]; the mask test is paid
-      // only on the diagonal
-      auto softmax_grad = [&](auto mask_c) {
-        constexpr bool kMask = decltype(mask_c)::value;
-        const int key_rel = kw0 + n - qs_pos - 4 * h;  // key is masked for row (8j + 4h + t) iff key_rel > 8j + t
+    };
+    // softmax_grad(): P = exp2(S*c - lse*log2e), dS = P * (dP - delta) [already in the accumulator]; the mask test
+    // is compiled in only for sub-blocks on the diagonal.
+    auto softmax_grad = [&](int sb, f32x16& s_acc, f32x16& dp_acc, auto mask_c) {
+      constexpr bool kMask = decltype(mask_c)::value;
+      const int qs_pos = a.q_offset + q0 + 32 * sb;
+      const int key_rel = kw0 + n - qs_pos - 4 * h;  // key is masked for row (8j + 4h + t) iff key_rel > 8j + t
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
+      for (int j = 0; j < 4; ++j) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int i = 4 * j + t;
-            float pv = fast_exp2(s_acc[i] * c - l4[t]);
-            if constexpr (kMask) {
-              if (key_rel > 8 * j + t) pv = 0.f;
-            }
-            s_acc[i] = pv;
-            dp_acc[i] = pv * dp_acc[i];
+        for (int t = 0; t < 4; ++t) {
+          const int i = 4 * j + t;
+          float pv = fast_exp2(s_acc[i] * c - l4[t]);
+          if constexpr (kMask) {
+            if (key_rel > 8 * j + t) pv = 0.f;
           }
+          s_acc[i] = pv;
+          dp_acc[i] = pv * dp_acc[i];
         }
-      };
-      if (a.causal && kw0 + 31 > qs_pos) softmax_grad(std::true_type{});
-      else softmax_grad(std::false_type{});
+      }
+    };
+    // accumulate(): the transposed products dV^T += dO^T P and dK^T += Q^T dS (lane = key, registers = 4 consecutive
+    // d, which is what lets the epilogue write whole 16-byte pieces of a row); P / dS come from the registers,
+    // dO^T / Q^T from the row-major LDS tiles through transposing reads.
+    auto accumulate = [&](int sb, const f32x16& s_acc, const f32x16& dp_acc) {
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
         // registers 8cc+4jj+t hold queries 32sb + 16cc + 8jj + 4h + t: fetch dO / Q rows in that order
@@ -266,11 +268,38 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
           const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
           const bf16x8 dof = lds_read_tr_pair(&sdO[qr * LDQ + col], LDQ);
           const bf16x8 qf = lds_read_tr_pair(&sQ[qr * LDQ + col], LDQ);
-          // transposed products dV^T = dO^T P and dK^T = Q^T dS: lane = key, registers = 4 consecutive d,
-          // which is what lets the epilogue write whole 16-byte pieces of a row
           dv_acc[db] = mfma32(dof, pf, dv_acc[db]);
           dk_acc[db] = mfma32(qf, dsf, dk_acc[db]);
         }
+      }
+    };
+
+    const bool off_diagonal = kPipelineTrip && BM == 64 && (!a.causal || kw0 + 31 <= a.q_offset + q0);
+    if (has_next && !off_diagonal) prefetch();
+    if (off_diagonal) {
+      // Every pair of this trip is visible to this wave (all trips off the diagonal): straight-line code in an order
+      // that lets the wave's own phases overlap -- the matrix pipe works on the second sub-block's S / dP while the
+      // vector pipe does the first one's softmax, and on the first one's dV / dK during the second one's softmax.
+      f32x16 s0, d0, s1, d1;
+      products(0, s0, d0);
+      products(1, s1, d1);
+      __builtin_amdgcn_sched_barrier(0);
+      softmax_grad(0, s0, d0, std::false_type{});
+      accumulate(0, s0, d0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (has_next) prefetch();  // issued here, not at the top of the trip: its registers are free until now
+      softmax_grad(1, s1, d1, std::false_type{});
+      accumulate(1, s1, d1);
+    } else {
+#pragma unroll
+      for (int sb = 0; sb < BM / 32; ++sb) {
+        const int qs_pos = a.q_offset + q0 + 32 * sb;       // position of the sub-block's first query
+        if (a.causal && kw0 > qs_pos + 31) continue;        // every (query, key) pair of this block is masked
+        f32x16 s_acc, dp_acc;
+        products(sb, s_acc, dp_acc);
+        if (a.causal && kw0 + 31 > qs_pos) softmax_grad(sb, s_acc, dp_acc, std::true_type{});
+        else softmax_grad(sb, s_acc, dp_acc, std::false_type{});
+        accumulate(sb, s_acc, dp_acc);
       }
     }
     buf_off ^= static_cast<uint32_t>(C::kBufBytes);
