@@ -153,10 +153,11 @@ class RingBench:
                           want_dkv=False)
 
     def step_batched(self):
-        ops = self.ops
+        # forward, then the backward as one call: the dQ kernel computes delta = sum_d dO * O in its prologue and the
+        # dK/dV kernel follows it
         self.forward_batched()
-        ops.attn_bwd_preprocess(self.do, self.out, delta=self.delta_b)
-        self.backward_kernel_batched()
+        self.ops.attn_bwd(self.do, self.q, self.k, self.v, self.lse_b, self.delta_b, self.scale, True, 0, self.dq_b,
+                          self.dk_b, self.dv_b, out=self.out)
 
     # -- the same work in the reference's shape: one launch per ring step (block + fused merge)
     def step_per_ring_step(self):

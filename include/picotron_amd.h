@@ -170,6 +170,18 @@ int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, cons
                   void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
                   void* stream);
 
+/* replaces: ring_attention_backward  context_parallel.py:130-155 as ONE call, delta = sum_d dO * O (:145) included.
+ * Same arguments as pico_attn_bwd plus the forward output `out` (addressed by o_stride like dout, dtype out_dtype);
+ * `delta` is an OUTPUT here: [B,Hq,Sq] fp32, written with the row sums.  With a bf16 `out` and a wanted dq the dQ
+ * kernel computes delta in its prologue and runs before the dK/dV kernel (one launch and one pass over dO and O
+ * less than pico_attn_bwd_preprocess + pico_attn_bwd); otherwise the pre-pass is enqueued internally.
+ */
+int pico_attn_bwd_fused(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
+                        const void* dout, const void* out, int out_dtype, const float* lse, float* delta,
+                        void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate,
+                        void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
+                        void* stream);
+
 /* fp32 -> bf16/fp32 conversion with layout change: src [B,H,S,D] contiguous fp32,
  * dst addressed by dst_stride (b,h,s).  Used to hand dq_acc back in the dtype / layout of q.
  * No counterpart in the reference (autograd does the cast, context_parallel.py:110).

@@ -27,6 +27,8 @@ struct BwdParams {
   const __bf16* dout;
   const float* lse;
   const float* delta;
+  const __bf16* out;   // fused-delta mode of the dQ kernel: the forward output, addressed like dout
+  float* delta_w;      //   ... and where that kernel writes delta = sum_d dO * O for the dK/dV kernel
   void* dq;
   void* dk;
   void* dv;
@@ -371,7 +373,7 @@ struct DqCfg {
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
-template <int D, int NW, int KT>
+template <int D, int NW, int KT, bool kDelta>
 __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p) {
   using C = DqCfg<D, NW, KT>;
   constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK;
@@ -405,15 +407,32 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
                          span_bytes(a.Sq - row0, a.qs[2], D)), a.qs[2], lane);
     dt.issue(make_buffer(p.dout + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(row0) * a.os[2],
                          span_bytes(a.Sq - row0, a.os[2], D)), a.os[2], lane);
+    WaveTile<D> ot;
+    if constexpr (kDelta)
+      ot.issue(make_buffer(p.out + b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(row0) * a.os[2],
+                           span_bytes(a.Sq - row0, a.os[2], D)), a.os[2], lane);
+    const int64_t gi = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + qrow;
     if (qlive) {
-      const int64_t gi = (static_cast<int64_t>(b) * a.Hq + hq) * a.Sq + qrow;
       const float l = p.lse[gi];
       lse2 = (l == -INFINITY) ? INFINITY : l * kLog2e;  // a row that saw no key contributes nothing
-      delta = p.delta[gi];
+      if constexpr (!kDelta) delta = p.delta[gi];
     }
     unsigned char* region = smem_raw + wave * WaveTile<D>::kRegionBytes;
     qt.fragments(region, lane, qf);
     dt.fragments(region, lane, dof);
+    if constexpr (kDelta) {
+      // delta = sum_d dO * O of the lane's row (context_parallel.py:145): each half of the wave holds half of the
+      // row's columns in its fragments; the dK/dV kernel, launched after this one, reads the result from memory
+      bf16x8 of[D / 16];
+      ot.fragments(region, lane, of);
+      float part = 0.f;
+#pragma unroll
+      for (int s = 0; s < D / 16; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part += static_cast<float>(dof[s][e]) * static_cast<float>(of[s][e]);
+      delta = half_sum(part);
+      if (qlive && h == 0) p.delta_w[gi] = delta;
+    }
   }
 
   f32x16 dq[D / 32];
@@ -628,17 +647,22 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
   return PICO_OK;
 }
 
-template <int D, int NW, int KT>
-int launch_dq(const BwdParams& p, hipStream_t s) {
+template <int D, int NW, int KT, bool kDelta>
+int launch_dq_impl(const BwdParams& p, hipStream_t s) {
   using C = DqCfg<D, NW, KT>;
   static bool attr_set = false;
   if (!attr_set) {
-    if (int rc = set_lds(&attn_bwd_dq_kernel<D, NW, KT>, C::kLdsBytes, "pico_attn_bwd(dq)")) return rc;
+    if (int rc = set_lds(&attn_bwd_dq_kernel<D, NW, KT, kDelta>, C::kLdsBytes, "pico_attn_bwd(dq)")) return rc;
     attr_set = true;
   }
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
-  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, NW, KT>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, NW, KT, kDelta>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
   return PICO_OK;
+}
+
+template <int D, int NW, int KT>
+int launch_dq(const BwdParams& p, hipStream_t s) {
+  return p.out ? launch_dq_impl<D, NW, KT, true>(p, s) : launch_dq_impl<D, NW, KT, false>(p, s);
 }
 
 }  // namespace
@@ -670,71 +694,114 @@ extern "C" int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* 
   return check_launch("pico_attn_bwd_preprocess");
 }
 
-extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
-                             const float* lse, const float* delta, void* dq, const int64_t* dq_stride, int dq_dtype,
-                             int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
-                             int dkv_accumulate, void* stream) {
-  if (int rc = check_attn_desc("pico_attn_bwd", desc)) return rc;
+namespace {
+
+// Shared body of pico_attn_bwd and pico_attn_bwd_fused.  With `out` (bf16 forward output) the dQ kernel computes
+// delta itself, writes it to `delta_w`, and runs BEFORE the dK/dV kernel, which reads it from there.
+int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
+            const float* lse, const float* delta, const void* out, float* delta_w, void* dq, const int64_t* dq_stride,
+            int dq_dtype, int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
+            int dkv_accumulate, void* stream) {
   if ((dkv_dtype != PICO_BF16 && dkv_dtype != PICO_F32) || (dq_dtype != PICO_BF16 && dq_dtype != PICO_F32))
-    return fail(PICO_ERR_DTYPE, "pico_attn_bwd: gradient dtype codes %d / %d not supported", dq_dtype, dkv_dtype);
+    return fail(PICO_ERR_DTYPE, "%s: gradient dtype codes %d / %d not supported", fn, dq_dtype, dkv_dtype);
   if ((dkv_accumulate && dkv_dtype != PICO_F32) || (dq_accumulate && dq_dtype != PICO_F32))
-    return fail(PICO_ERR_DTYPE, "pico_attn_bwd: accumulate needs fp32 gradients");
+    return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
   if (desc->B == 0) return PICO_OK;
   // a gradient that is not wanted is passed as NULL and its kernel is skipped
   const bool want_dq = dq != nullptr, want_dkv = dk != nullptr || dv != nullptr;
-  if (want_dkv && (!dk || !dv)) return fail(PICO_ERR_NULL, "pico_attn_bwd: dk and dv must be given together");
+  if (want_dkv && (!dk || !dv)) return fail(PICO_ERR_NULL, "%s: dk and dv must be given together", fn);
   const bool have_q = desc->Sq > 0 && want_dq, have_k = desc->Sk > 0 && want_dkv;
   if (((have_q || have_k) && desc->Sq > 0 && (!q || !dout || !lse || !delta)) ||
       ((have_q || have_k) && desc->Sk > 0 && (!k || !v)))
-    return fail(PICO_ERR_NULL, "pico_attn_bwd: q, k, v, dout, lse and delta are required");
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) || !aligned16(dv))
-    return fail(PICO_ERR_ALIGN, "pico_attn_bwd: q, k, v, dout, dq, dk and dv must be 16-byte aligned");
+    return fail(PICO_ERR_NULL, "%s: q, k, v, dout, lse and delta are required", fn);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) ||
+      !aligned16(dv) || !aligned16(out))
+    return fail(PICO_ERR_ALIGN, "%s: q, k, v, dout, out, dq, dk and dv must be 16-byte aligned", fn);
   BwdParams p;
   p.a = make_params(desc, q, k, v);
   p.dout = static_cast<const __bf16*>(dout);
   p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.out = static_cast<const __bf16*>(out);
+  p.delta_w = delta_w;
   p.dq_f32 = dq_dtype == PICO_F32;
   p.dq_accumulate = dq_accumulate != 0;
   p.dkv_f32 = dkv_dtype == PICO_F32;
   p.dkv_accumulate = dkv_accumulate != 0;
-  auto strides = [&](const int64_t* given, int heads, int seq, int64_t (&out)[3], int align) -> bool {
+  p.pair_ktiles = 0;
+  auto strides = [&](const int64_t* given, int heads, int seq, int64_t (&st)[3], int align) -> bool {
     if (given) {
       for (int i = 0; i < 3; ++i) {
         if (given[i] < 0 || given[i] % align != 0) return false;
-        out[i] = given[i];
+        st[i] = given[i];
       }
     } else {
-      out[2] = desc->D;
-      out[1] = static_cast<int64_t>(seq) * desc->D;
-      out[0] = out[1] * heads;
+      st[2] = desc->D;
+      st[1] = static_cast<int64_t>(seq) * desc->D;
+      st[0] = st[1] * heads;
     }
     return true;
   };
   if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, p.dq_f32 ? 4 : 8) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 8))
-    return fail(PICO_ERR_STRIDE, "pico_attn_bwd: dq strides must be non-negative multiples of 4 (fp32) or 8 (bf16), dk/dv strides of 8");
+    return fail(PICO_ERR_STRIDE, "%s: dq strides must be non-negative multiples of 4 (fp32) or 8 (bf16), dk/dv strides of 8", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int rc = PICO_OK;
-  if (have_k) {
+  auto run_dkdv = [&]() -> int {
+    if (!have_k) return PICO_OK;
     // without queries the dK/dV kernel still runs: it writes (or adds) zeros
-    rc = desc->D == 64 ? launch_dkdv<64>(p, s) : launch_dkdv<128>(p, s);
-    if (rc) return rc;
-    if (int lrc = check_launch("pico_attn_bwd(dk/dv)")) return lrc;
-  }
-  if (have_q) {
+    if (int rc = desc->D == 64 ? launch_dkdv<64>(p, s) : launch_dkdv<128>(p, s)) return rc;
+    return check_launch("pico_attn_bwd(dk/dv)");
+  };
+  auto run_dq = [&]() -> int {
+    if (!have_q) return PICO_OK;
     // without keys the dQ kernel still runs: it writes (or adds) zeros
+    int rc;
+    const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     if (desc->D == 64) {
-      const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
       auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
       if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
       else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
       else rc = launch_dq<64, 2, 64>(p, s);
     } else {
-      const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
       if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch_dq<128, 8, 64>(p, s);
       else rc = launch_dq<128, 4, 64>(p, s);
     }
     if (rc) return rc;
-    if (int lrc = check_launch("pico_attn_bwd(dq)")) return lrc;
+    return check_launch("pico_attn_bwd(dq)");
+  };
+  if (p.out) {  // the dQ kernel produces delta for the dK/dV kernel
+    if (int rc = run_dq()) return rc;
+    return run_dkdv();
   }
-  return PICO_OK;
+  if (int rc = run_dkdv()) return rc;
+  return run_dq();
+}
+
+}  // namespace
+
+extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
+                             const float* lse, const float* delta, void* dq, const int64_t* dq_stride, int dq_dtype,
+                             int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
+                             int dkv_accumulate, void* stream) {
+  if (int rc = check_attn_desc("pico_attn_bwd", desc)) return rc;
+  return run_bwd("pico_attn_bwd", desc, q, k, v, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype, dq_accumulate,
+                 dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
+}
+
+extern "C" int pico_attn_bwd_fused(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
+                                   const void* dout, const void* out, int out_dtype, const float* lse, float* delta,
+                                   void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate, void* dk, void* dv,
+                                   const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate, void* stream) {
+  if (int rc = check_attn_desc("pico_attn_bwd_fused", desc)) return rc;
+  if (out_dtype != PICO_BF16 && out_dtype != PICO_F32)
+    return fail(PICO_ERR_DTYPE, "pico_attn_bwd_fused: out dtype code %d not supported", out_dtype);
+  if (desc->B == 0) return PICO_OK;
+  if (desc->Sq > 0 && (!out || !delta)) return fail(PICO_ERR_NULL, "pico_attn_bwd_fused: out and delta are required");
+  // delta inside the dQ kernel needs that kernel to run and a bf16 out; otherwise the pre-pass computes it
+  const bool in_kernel = out_dtype == PICO_BF16 && dq != nullptr && desc->Sq > 0;
+  if (!in_kernel) {
+    if (int rc = pico_attn_bwd_preprocess(desc, dout, out, out_dtype, delta, nullptr, stream)) return rc;
+    return run_bwd("pico_attn_bwd_fused", desc, q, k, v, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype,
+                   dq_accumulate, dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
+  }
+  return run_bwd("pico_attn_bwd_fused", desc, q, k, v, dout, lse, delta, out, delta, dq, dq_stride, dq_dtype, dq_accumulate,
+                 dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
 }

@@ -82,8 +82,8 @@ class FlashAttnFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dout):
         q, k, v, out, lse = ctx.saved_tensors
-        delta = ops.attn_bwd_preprocess(dout, out)
-        # gradients come back in the dtype and memory layout of their inputs: no accumulation buffer, no cast pass
-        dq, dk, dv = ops.attn_bwd(dout, q, k, v, lse, delta, ctx.sm_scale, ctx.causal, 0, dq_dtype=q.dtype, dq_like=q,
-                                  dkv_dtype=k.dtype)
+        # delta = sum_d dout * out is computed inside the call; gradients come back in the dtype and memory layout of
+        # their inputs: no accumulation buffer, no cast pass
+        dq, dk, dv = ops.attn_bwd(dout, q, k, v, lse, None, ctx.sm_scale, ctx.causal, 0, dq_dtype=q.dtype, dq_like=q,
+                                  dkv_dtype=k.dtype, out=out)
         return dq, dk, dv, None, None

@@ -245,21 +245,36 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
              dq: Optional[torch.Tensor] = None, dk: Optional[torch.Tensor] = None, dv: Optional[torch.Tensor] = None,
              dq_accumulate: bool = False, dkv_accumulate: bool = False, dq_dtype=torch.float32,
              dkv_dtype=torch.float32, dq_like: Optional[torch.Tensor] = None, want_dq: bool = True,
-             want_dkv: bool = True, side_stream: Optional["torch.cuda.Stream"] = None):
+             want_dkv: bool = True, side_stream: Optional["torch.cuda.Stream"] = None,
+             out: Optional[torch.Tensor] = None):
     """Gradients of one attention block; returns (dq [B,Hq,Sq,D], dk, dv [B,Hkv,Sk,D]).
 
     Buffers that are passed in are written in place (fp32 ones can be accumulated into: the running dq of a
     rank and the travelling dk / dv of the ring); missing ones are allocated in the requested dtype, dq with
     the strides of `dq_like` if given.  want_dq / want_dkv = False skips that gradient (and its kernel).
+    With `out` (the forward output) `delta` may be None or a buffer to fill: the row sums delta = sum_d dout * out are
+    then computed inside the call (by the dQ kernel itself when out is bf16 and dq is wanted), as in the reference's
+    ring_attention_backward, instead of by a separate attn_bwd_preprocess.
     With `side_stream` the dQ kernel is enqueued there and the dK/dV kernel on the current stream (the two are
     independent); the current stream waits for both.  Measured on MI355X it is a wash at the benchmark shape
     (+3 % on one box, -4 % on another: the fork / join costs what the overlapped tails save), so nothing in
     this package turns it on by default.
     """
-    _dev(dout, q, k, v, lse, delta, dq, dk, dv)
+    _dev(dout, q, k, v, lse, delta, dq, dk, dv, out)
     q, k, v, dout = _attn_in(q, "q"), _attn_in(k, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
     B, Hq, Sq, D = q.shape
     Hkv, Sk = k.size(1), k.size(2)
+    if out is not None:
+        if side_stream is not None:
+            raise RuntimeError("attn_bwd: out= (delta computed by the dQ kernel) orders the two kernels; no side_stream")
+        if out.stride() != dout.stride():
+            out = _like_strided(out, dout)
+        if delta is None:
+            delta = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+        elif not (delta.is_contiguous() and delta.dtype == torch.float32 and delta.numel() == B * Hq * Sq):
+            raise RuntimeError("attn_bwd: delta must be contiguous fp32 [B,H,S]")
+    elif delta is None:
+        raise RuntimeError("attn_bwd: delta (or out, to compute it) is required")
     if dq is None and want_dq:
         if dq_accumulate:
             raise RuntimeError("attn_bwd: dq_accumulate=True needs an existing dq")
@@ -288,6 +303,14 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
     lse_c, delta_c = lse.contiguous(), delta.contiguous()
 
     def launch(dq_, dk_, dv_):
+        if out is not None:
+            check(_lib.lib().pico_attn_bwd_fused(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(out),
+                                                 _dt(out, "out"), _ptr(lse_c), _ptr(delta_c), _ptr(dq_), dqs,
+                                                 _dt(dq, "dq") if dq is not None else PICO_F32, int(dq_accumulate),
+                                                 _ptr(dk_), _ptr(dv_), dks,
+                                                 _dt(dk, "dk/dv") if dk is not None else PICO_F32, int(dkv_accumulate),
+                                                 _stream()))
+            return
         check(_lib.lib().pico_attn_bwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(dout), _ptr(lse_c), _ptr(delta_c),
                                        _ptr(dq_), dqs, _dt(dq, "dq") if dq is not None else PICO_F32, int(dq_accumulate),
                                        _ptr(dk_), _ptr(dv_), dks, _dt(dk, "dk/dv") if dk is not None else PICO_F32,

@@ -365,6 +365,29 @@ def test_attn_bwd_paired_key_tiles_match_unpaired(ops, device):
     assert rel_l2(whole[1][:1, :1], gk) <= 1e-2 and rel_l2(whole[2][:1, :1], gv) <= 1e-2 and rel_l2(whole[0][:1, :1], gq) <= 1e-2
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,q_offset", [
+    (2, 4, 4, 300, 300, 64, True, 0), (1, 4, 2, 128, 384, 128, True, 256), (1, 2, 1, 77, 203, 64, False, 0)])
+def test_attn_bwd_with_delta_computed_inside(ops, device, B, Hq, Hkv, Sq, Sk, D, causal, q_offset):
+    """attn_bwd(out=...) computes delta = sum_d dO * O itself (in the dQ kernel's prologue for a bf16 out, through the
+    pre-pass for an fp32 out or when dq is not wanted): same gradients as preprocess + attn_bwd, and delta is handed back."""
+    q, k, v = (t.to(device) for t in attn_inputs(B, Hq, Hkv, Sq, Sk, D, seed=92))
+    do = rnd(B, Hq, Sq, D, seed=93).to(torch.bfloat16).to(device)
+    scale = 1 / math.sqrt(D)
+    out, lse = ops.attn_fwd(q, k, v, scale, causal, q_offset)
+    delta = ops.attn_bwd_preprocess(do, out)
+    ref = ops.attn_bwd(do, q, k, v, lse, delta, scale, causal, q_offset)
+    want = (do.float() * out.float()).sum(-1)
+    for out_arg in (out, out.float()):
+        d2 = torch.full_like(delta, float("nan"))
+        got = ops.attn_bwd(do, q, k, v, lse, d2, scale, causal, q_offset, out=out_arg)
+        assert maxabs(d2, want) <= 1e-3 * max(1.0, want.abs().max().item())
+        for x, y in zip(got, ref):
+            assert rel_l2(x, y) <= 1e-4
+    # dq not wanted: the pre-pass supplies delta for the dK/dV kernel
+    _, dk, dv = ops.attn_bwd(do, q, k, v, lse, None, scale, causal, q_offset, out=out, want_dq=False)
+    assert rel_l2(dk, ref[1]) <= 1e-4 and rel_l2(dv, ref[2]) <= 1e-4
+
+
 def test_attn_rejects_unsupported_layouts(ops, device):
     """Error behaviour of the boundary: gradient rows that are not 16-byte aligned raise, nothing is launched."""
     B, H, S, D = 1, 2, 64, 64
