@@ -41,7 +41,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0   # MI355X dense bf16
 HBM_PEAK_GBS = 8000.0
 # HBM bytes of one dK/dV launch at the bench shape, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a copy
 # kernel of known size (see profiles/); None until measured
-TRAFFIC_BYTES_DKDV = 103.8e6
+TRAFFIC_BYTES_DKDV = 107.8e6
 
 
 def parse():
