@@ -275,25 +275,19 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
     with torch.device("cuda"):
         model = Llama(cfg)
     model = model.to(torch.bfloat16)
-    params = [p for p in model.parameters()]
-    master = [p.detach().float().clone() for p in params]
-    for m in master:
-        m.grad = torch.zeros_like(m)
-    opt = torch.optim.AdamW(master, lr=3e-4, fused=True)
+    # fp32 master weights and AdamW moments; one fused pass per parameter tensor reads the bf16 gradient and rewrites
+    # the bf16 parameter (picotron_amd.optim.FusedAdamW over pico_adamw)
+    from picotron_amd.optim import FusedAdamW
+    opt = FusedAdamW(model.parameters(), lr=3e-4)
     ids, tgt = synthetic_batch(cfg.vocab_size, mbs, seq, seed=0)
     ids, tgt = ids.cuda(), tgt.cuda()
 
     def step():
-        for p in params:
-            p.grad = None
+        opt.zero_grad()
         logits = model(input_ids=ids)
         loss = F.cross_entropy(logits.view(mbs * seq, -1).float(), tgt.reshape(-1), reduction="mean")
         loss.backward()
-        with torch.no_grad():
-            torch._foreach_copy_([m.grad for m in master], [p.grad for p in params])
         opt.step()
-        with torch.no_grad():
-            torch._foreach_copy_([p.data for p in params], master)
         return loss
 
     for _ in range(warmup):
@@ -309,8 +303,9 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
     fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, seq)
     res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
            "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
-           "note": "attention / RMSNorm / RoPE / SwiGLU on the HIP kernels; projections, CE and AdamW on torch"}
-    del model, params, master, opt
+           "note": "attention / RMSNorm / RoPE / SwiGLU / AdamW (fp32 master weights and moments) on the HIP kernels; "
+                   "projections and CE on torch"}
+    del model, opt
     torch.cuda.empty_cache()
     return res
 

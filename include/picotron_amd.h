@@ -190,6 +190,20 @@ int pico_convert_f32(const float* src, void* dst, int64_t B, int64_t H, int64_t 
                      int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_stride_s,
                      int dst_dtype, void* stream);
 
+/* ------------------------------------------------------------------ optimizer step
+ * replaces: torch.optim.AdamW(model.parameters(), lr).step()  train.py:204-209,240  for low-precision parameters
+ *           with fp32 state: the reference keeps the AdamW state in the parameter dtype; here master weights and
+ *           both moments are fp32 and the bf16 parameter is rewritten from the master weight in the same pass.
+ * Same order of operations as torch's AdamW (decoupled weight decay, no amsgrad):
+ *   p *= 1 - lr*wd;  m += (g - m)*(1 - beta1);  v = v*beta2 + g*g*(1 - beta2);
+ *   p -= lr/bc1 * m / (sqrt(v)/sqrt(bc2) + eps),  bc_i = 1 - beta_i^step,  g = grad * grad_scale.
+ * param_lp: [n] bf16, written (may be NULL); master, exp_avg, exp_avg_sq: [n] fp32, updated in place;
+ * grad: [n] of grad_dtype (PICO_BF16 or PICO_F32); step counts from 1.
+ */
+int pico_adamw(void* param_lp, float* master, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
+               int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step,
+               float grad_scale, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

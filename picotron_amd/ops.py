@@ -344,3 +344,24 @@ def convert_f32(src: torch.Tensor, dtype, like: Optional[torch.Tensor] = None, b
     check(_lib.lib().pico_convert_f32(_ptr(src), _ptr(dst), B, H, S, D, dst.stride(0), dst.stride(1), dst.stride(2),
                                       _DT[dtype], _stream()))
     return dst
+
+
+def adamw_(param_lp: Optional[torch.Tensor], master: torch.Tensor, grad: torch.Tensor, exp_avg: torch.Tensor,
+           exp_avg_sq: torch.Tensor, step: int, lr: float, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8,
+           weight_decay: float = 0.01, grad_scale: float = 1.0) -> None:
+    """In-place AdamW step on fp32 (master, exp_avg, exp_avg_sq) from a bf16 / fp32 gradient; rewrites the bf16
+    parameter `param_lp` (if given) from the new master weight.  `step` counts from 1."""
+    _dev(param_lp, master, grad, exp_avg, exp_avg_sq)
+    n = master.numel()
+    for t, what in ((master, "master"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+        if t.dtype != torch.float32 or not t.is_contiguous() or t.numel() != n:
+            raise RuntimeError(f"adamw_: {what} must be a contiguous fp32 tensor of {n} elements")
+    if not grad.is_contiguous() or grad.numel() != n:
+        grad = grad.contiguous()
+        if grad.numel() != n:
+            raise RuntimeError("adamw_: grad has the wrong number of elements")
+    if param_lp is not None and (param_lp.dtype != torch.bfloat16 or not param_lp.is_contiguous() or param_lp.numel() != n):
+        raise RuntimeError("adamw_: param_lp must be a contiguous bf16 tensor of the same size")
+    check(_lib.lib().pico_adamw(_ptr(param_lp), _ptr(master), _ptr(grad), _dt(grad, "grad"), _ptr(exp_avg), _ptr(exp_avg_sq),
+                                n, float(lr), float(beta1), float(beta2), float(eps), float(weight_decay), int(step),
+                                float(grad_scale), _stream()))

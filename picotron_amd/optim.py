@@ -1,0 +1,57 @@
+"""AdamW for bf16 parameters with fp32 master weights and moments, one fused HIP pass per parameter tensor.
+
+The reference builds ``torch.optim.AdamW(model.parameters(), lr)`` (``train.py:204-209``; its ``fused`` switch is
+dead code) and so keeps the optimizer state in the parameter dtype.  Here the state is fp32: a master copy of every
+parameter plus both moments, laid out in three flat buffers, and ``step()`` reads each bf16 gradient once and rewrites
+the bf16 parameter from the updated master weight in the same kernel (``pico_adamw``) -- no cast passes."""
+from __future__ import annotations
+
+from typing import Iterable
+
+import torch
+
+from . import ops
+
+
+class FusedAdamW:
+    def __init__(self, params: Iterable[torch.nn.Parameter], lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
+                 weight_decay: float = 1e-2):
+        self.params = [p for p in params if p.requires_grad]
+        if not self.params:
+            raise ValueError("FusedAdamW: no parameters")
+        for p in self.params:
+            if not p.is_cuda or p.dtype not in (torch.bfloat16, torch.float32) or not p.is_contiguous():
+                raise RuntimeError("FusedAdamW: parameters must be contiguous bf16 / fp32 tensors on the GPU")
+        self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
+        self.step_count = 0
+        dev = self.params[0].device
+        # every tensor starts on a multiple of 8 elements so that all kernel accesses are 16-byte aligned
+        self.offsets, total = [], 0
+        for p in self.params:
+            self.offsets.append(total)
+            total += (p.numel() + 7) // 8 * 8
+        self.master = torch.zeros(total, dtype=torch.float32, device=dev)
+        self.exp_avg = torch.zeros(total, dtype=torch.float32, device=dev)
+        self.exp_avg_sq = torch.zeros(total, dtype=torch.float32, device=dev)
+        for p, off in zip(self.params, self.offsets):
+            self.master[off:off + p.numel()].copy_(p.detach().reshape(-1))
+
+    def zero_grad(self, set_to_none: bool = True):
+        for p in self.params:
+            if set_to_none:
+                p.grad = None
+            elif p.grad is not None:
+                p.grad.zero_()
+
+    @torch.no_grad()
+    def step(self, grad_scale: float = 1.0):
+        self.step_count += 1
+        for p, off in zip(self.params, self.offsets):
+            if p.grad is None:
+                continue
+            n = p.numel()
+            ops.adamw_(p if p.dtype == torch.bfloat16 else None, self.master[off:off + n], p.grad,
+                       self.exp_avg[off:off + n], self.exp_avg_sq[off:off + n], self.step_count, self.lr, self.betas[0],
+                       self.betas[1], self.eps, self.weight_decay, grad_scale)
+            if p.dtype == torch.float32:
+                p.copy_(self.master[off:off + n].view_as(p))

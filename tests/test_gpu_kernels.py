@@ -431,3 +431,43 @@ def test_bad_head_dim_reports_error(ops, device):
     q = torch.zeros(1, 1, 8, 32, dtype=torch.bfloat16, device=device)
     with pytest.raises(RuntimeError, match="head_dim"):
         ops.attn_fwd(q, q, q, 1.0, True)
+
+
+@pytest.mark.parametrize("n,grad_dtype", [(8 * 1024 + 3, torch.bfloat16), (4096, torch.float32), (5, torch.bfloat16)])
+def test_adamw_kernel_against_oracle(ops, device, n, grad_dtype):
+    """pico_adamw over four steps against oracle.optim.master_step: fp32 states to a few ulp, the bf16 parameter is the
+    rounded master weight."""
+    from oracle import optim as OO
+    g = torch.Generator().manual_seed(11)
+    master = torch.randn(n, generator=g)
+    m, v = torch.zeros(n), torch.zeros(n)
+    d_master, d_m, d_v = master.to(device), m.to(device), v.to(device)
+    d_p = torch.empty(n, dtype=torch.bfloat16, device=device)
+    for step in range(1, 5):
+        grad = (torch.randn(n, generator=g) * 0.05 * step).to(grad_dtype)
+        ops.adamw_(d_p, d_master, grad.to(device), d_m, d_v, step, 2e-3, 0.9, 0.95, 1e-8, 0.1)
+        master, m, v, p_lp = OO.master_step(master, grad, m, v, step, 2e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+        assert maxabs(d_master, master) <= 2e-6 * max(1.0, master.abs().max().item())
+        assert maxabs(d_m, m) <= 1e-6 and maxabs(d_v, v) <= 1e-6
+        assert torch.equal(d_p.cpu(), d_master.cpu().to(torch.bfloat16))
+
+
+def test_fused_adamw_trains_like_torch_adamw_on_master_weights(device):
+    """picotron_amd.optim.FusedAdamW on bf16 parameters follows torch.optim.AdamW run on fp32 copies fed the same
+    bf16 gradients."""
+    from picotron_amd.optim import FusedAdamW
+    torch.manual_seed(3)
+    ps = [torch.nn.Parameter(torch.randn(33, 20, device=device).to(torch.bfloat16)), torch.nn.Parameter(torch.randn(7, device=device).to(torch.bfloat16))]
+    ref = [torch.nn.Parameter(p.detach().float().clone()) for p in ps]
+    opt, ropt = FusedAdamW(ps, lr=1e-2, weight_decay=0.02), torch.optim.AdamW(ref, lr=1e-2, weight_decay=0.02)
+    for _ in range(3):
+        for p, r in zip(ps, ref):
+            p.grad = torch.randn_like(p)
+            r.grad = p.grad.float()
+        opt.step()
+        ropt.step()
+    for p, r, off in zip(ps, ref, opt.offsets):
+        mine = opt.master[off:off + p.numel()].view_as(r)
+        assert maxabs(mine, r.detach()) <= 1e-5
+        assert torch.equal(p.detach().cpu(), mine.to(torch.bfloat16).cpu())
+        assert maxabs(p.detach().float(), r.detach()) <= 2 ** -8 * r.detach().abs().max().item()

@@ -138,3 +138,24 @@ def test_swiglu_forward_and_backward():
     z = torch.zeros(1, dtype=torch.float64)
     dg0, du0 = layers.swiglu_backward(torch.ones(1, dtype=torch.float64), z, torch.full((1,), 3.0, dtype=torch.float64))
     assert dg0.item() == pytest.approx(1.5) and du0.item() == 0.0
+
+
+def test_adamw_step_matches_torch_adamw():
+    """oracle.optim.adamw_step against torch.optim.AdamW (the routine the reference calls, train.py:204-209) over
+    five steps with changing gradients, in fp64 and fp32; a wrong bias correction, a coupled weight decay or a
+    swapped beta shows up in the first step already."""
+    from oracle import optim as OO
+    for dtype, tol in ((torch.float64, 1e-12), (torch.float32, 2e-6)):
+        g = torch.Generator().manual_seed(7)
+        p0 = torch.randn(257, generator=g, dtype=torch.float64).to(dtype)
+        ref = torch.nn.Parameter(p0.clone())
+        opt = torch.optim.AdamW([ref], lr=3e-3, betas=(0.85, 0.97), eps=1e-7, weight_decay=0.05)
+        p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+        for step in range(1, 6):
+            grad = torch.randn(257, generator=g, dtype=torch.float64).to(dtype) * (0.1 * step)
+            ref.grad = grad.clone()
+            opt.step()
+            p, m, v = OO.adamw_step(p, grad, m, v, step, 3e-3, 0.85, 0.97, 1e-7, 0.05)
+            assert (p - ref.detach()).abs().max().item() <= tol * max(1.0, p.abs().max().item())
+        st = opt.state[ref]
+        assert (m - st["exp_avg"]).abs().max().item() <= tol and (v - st["exp_avg_sq"]).abs().max().item() <= tol
