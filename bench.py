@@ -277,6 +277,7 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
     model = model.to(torch.bfloat16)
     # fp32 master weights and AdamW moments; one fused pass per parameter tensor reads the bf16 gradient and rewrites
     # the bf16 parameter (picotron_amd.optim.FusedAdamW over pico_adamw)
+    from picotron_amd.functional import cross_entropy
     from picotron_amd.optim import FusedAdamW
     opt = FusedAdamW(model.parameters(), lr=3e-4)
     ids, tgt = synthetic_batch(cfg.vocab_size, mbs, seq, seed=0)
@@ -285,7 +286,7 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
     def step():
         opt.zero_grad()
         logits = model(input_ids=ids)
-        loss = F.cross_entropy(logits.view(mbs * seq, -1).float(), tgt.reshape(-1), reduction="mean")
+        loss = cross_entropy(logits.view(mbs * seq, -1), tgt.reshape(-1))
         loss.backward()
         opt.step()
         return loss
@@ -303,8 +304,8 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
     fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, seq)
     res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
            "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
-           "note": "attention / RMSNorm / RoPE / SwiGLU / AdamW (fp32 master weights and moments) on the HIP kernels; "
-                   "projections and CE on torch"}
+           "note": "attention / RMSNorm / RoPE / SwiGLU / cross-entropy / AdamW (fp32 master weights and moments) on the HIP "
+                   "kernels; embedding, projections and residual adds on torch"}
     del model, opt
     torch.cuda.empty_cache()
     return res

@@ -190,6 +190,22 @@ int pico_convert_f32(const float* src, void* dst, int64_t B, int64_t H, int64_t 
                      int64_t dst_stride_b, int64_t dst_stride_h, int64_t dst_stride_s,
                      int dst_dtype, void* stream);
 
+/* ------------------------------------------------------------------ loss
+ * replaces: F.cross_entropy(outputs.view(S*B, V), target_ids, reduction='mean')  train.py:46-49  and its autograd.
+ * logits: [rows, vocab] with row pitch ld (elements; a multiple of 8 for bf16, 4 for fp32), dtype `dtype`;
+ * targets: [rows] int64, each in [0, vocab) or equal to ignore_index (torch's default is -100).
+ * forward : loss[r] = logsumexp(logits[r]) - logits[r][target[r]] (0 for an ignored row) and lse[r], both fp32 [rows].
+ *           The mean over the rows that are not ignored is left to the caller (one small reduction).
+ * backward: dlogits[r][j] = (exp(logits[r][j] - lse[r]) - (j == target[r])) * scale[0], 0 for an ignored row;
+ *           `scale` is a DEVICE pointer to one float (upstream gradient / number of rows that count), so no host
+ *           synchronisation is needed; dlogits has pitch dld and may alias logits.
+ */
+int pico_cross_entropy_fwd(const void* logits, const int64_t* targets, float* loss, float* lse, int64_t rows,
+                           int64_t vocab, int64_t ld, int64_t ignore_index, int dtype, void* stream);
+int pico_cross_entropy_bwd(const void* logits, const int64_t* targets, const float* lse, const float* scale,
+                           void* dlogits, int64_t rows, int64_t vocab, int64_t ld, int64_t dld, int64_t ignore_index,
+                           int dtype, void* stream);
+
 /* ------------------------------------------------------------------ optimizer step
  * replaces: torch.optim.AdamW(model.parameters(), lr).step()  train.py:204-209,240  for low-precision parameters
  *           with fp32 state: the reference keeps the AdamW state in the parameter dtype; here master weights and

@@ -86,3 +86,24 @@ def swiglu_backward(dy, gate, up):
     g, u, d = gate.to(acc), up.to(acc), dy.to(acc)
     sg = torch.sigmoid(g)
     return d * u * sg * (1 + g * (1 - sg)), d * g * sg
+
+
+def cross_entropy(logits: torch.Tensor, targets: torch.Tensor, ignore_index: int = -100):
+    """Mean cross-entropy as ``train.py:46-49`` computes it (``F.cross_entropy(..., reduction='mean')``), written out:
+    loss_r = logsumexp(logits_r) - logits_r[target_r]; mean over the rows whose target is not ignore_index.
+    Returns (loss, per-row logsumexp).  Pinned against ``F.cross_entropy`` in tests/test_oracle_layers.py."""
+    x = logits.float()
+    lse = torch.logsumexp(x, dim=-1)
+    keep = targets != ignore_index
+    picked = x.gather(1, targets.clamp(min=0).unsqueeze(1)).squeeze(1)
+    rows = torch.where(keep, lse - picked, torch.zeros_like(lse))
+    return rows.sum() / keep.sum().clamp(min=1), lse
+
+
+def cross_entropy_backward(logits: torch.Tensor, targets: torch.Tensor, grad_out: float = 1.0, ignore_index: int = -100):
+    """d loss / d logits = (softmax - onehot) * grad_out / count on kept rows, 0 on ignored ones."""
+    x = logits.float()
+    keep = targets != ignore_index
+    p = torch.softmax(x, dim=-1)
+    p[torch.arange(x.size(0)), targets.clamp(min=0)] -= 1.0
+    return p * keep.unsqueeze(1) * (grad_out / keep.sum().clamp(min=1))

@@ -40,6 +40,8 @@ SIGNATURES = {
     "pico_attn_bwd_preprocess": (c_int, [POINTER(AttnDesc), _P, _P, c_int, _P, _P, _P]),
     "pico_attn_bwd": (c_int, [POINTER(AttnDesc)] + [_P] * 6 + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int, _P]),
     "pico_attn_bwd_fused": (c_int, [POINTER(AttnDesc)] + [_P] * 5 + [c_int, _P, _P] + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int, _P]),
+    "pico_cross_entropy_fwd": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, c_int, _P]),
+    "pico_cross_entropy_bwd": (c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, c_int, _P]),
     "pico_adamw": (c_int, [_P, _P, _P, c_int, _P, _P, _I64] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
     "pico_convert_f32": (c_int, [_P, _P] + [_I64] * 7 + [c_int, _P]),
 }

@@ -17,7 +17,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(CSRC, "build")
 LIB = os.path.join(HERE, "libpicotron_amd.so")
 
-SOURCES = ["common.hip", "norm.hip", "pointwise.hip", "optim.hip", "attn_fwd.hip", "attn_bwd.hip"]
+SOURCES = ["common.hip", "norm.hip", "pointwise.hip", "optim.hip", "loss.hip", "attn_fwd.hip", "attn_bwd.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-munsafe-fp-atomics",
     # packed fp32 VALU forms are kept out of the generated code on purpose

@@ -87,3 +87,28 @@ class FlashAttnFunc(torch.autograd.Function):
         dq, dk, dv = ops.attn_bwd(dout, q, k, v, lse, None, ctx.sm_scale, ctx.causal, 0, dq_dtype=q.dtype, dq_like=q,
                                   dkv_dtype=k.dtype, out=out)
         return dq, dk, dv, None, None
+
+
+class CrossEntropyFunc(torch.autograd.Function):
+    """Mean cross-entropy of [rows, vocab] logits against int64 targets (``train.py:46-49``), fp32 loss.
+    The backward writes dlogits in the dtype of the logits in one pass; the upstream gradient and the 1 / count
+    factor reach the kernel through a device scalar, so nothing synchronises with the host."""
+
+    @staticmethod
+    def forward(ctx, logits, targets, ignore_index=-100):
+        loss_rows, lse = ops.cross_entropy_fwd(logits, targets, ignore_index)
+        count = (targets != ignore_index).sum().clamp(min=1).to(torch.float32)
+        ctx.save_for_backward(logits, targets, lse, count)
+        ctx.ignore_index = ignore_index
+        return loss_rows.sum() / count
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        logits, targets, lse, count = ctx.saved_tensors
+        scale = (grad_out.to(torch.float32) / count).reshape(1)
+        return ops.cross_entropy_bwd(logits, targets, lse, scale, ctx.ignore_index), None, None
+
+
+def cross_entropy(logits, targets, ignore_index: int = -100):
+    """Drop-in for ``F.cross_entropy(logits, targets, reduction='mean')`` on 2-D logits."""
+    return CrossEntropyFunc.apply(logits, targets, ignore_index)

@@ -365,3 +365,38 @@ def adamw_(param_lp: Optional[torch.Tensor], master: torch.Tensor, grad: torch.T
     check(_lib.lib().pico_adamw(_ptr(param_lp), _ptr(master), _ptr(grad), _dt(grad, "grad"), _ptr(exp_avg), _ptr(exp_avg_sq),
                                 n, float(lr), float(beta1), float(beta2), float(eps), float(weight_decay), int(step),
                                 float(grad_scale), _stream()))
+
+
+def _ce_check(logits: torch.Tensor, targets: torch.Tensor):
+    _dev(logits, targets)
+    if logits.dim() != 2 or logits.stride(1) != 1:
+        raise RuntimeError("cross_entropy: logits must be [rows, vocab] with a unit stride on vocab")
+    if targets.dtype != torch.int64 or not targets.is_contiguous() or targets.numel() != logits.size(0):
+        raise RuntimeError("cross_entropy: targets must be a contiguous int64 tensor with one entry per row")
+
+
+def cross_entropy_fwd(logits: torch.Tensor, targets: torch.Tensor, ignore_index: int = -100):
+    """Per-row loss and logsumexp, both fp32 [rows]."""
+    _ce_check(logits, targets)
+    rows, vocab = logits.shape
+    loss = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    lse = torch.empty(rows, dtype=torch.float32, device=logits.device)
+    check(_lib.lib().pico_cross_entropy_fwd(_ptr(logits), _ptr(targets), _ptr(loss), _ptr(lse), rows, vocab,
+                                            logits.stride(0) if rows else vocab, ignore_index, _dt(logits, "logits"), _stream()))
+    return loss, lse
+
+
+def cross_entropy_bwd(logits: torch.Tensor, targets: torch.Tensor, lse: torch.Tensor, scale: torch.Tensor,
+                      ignore_index: int = -100, inplace: bool = False) -> torch.Tensor:
+    """dlogits = (softmax(logits) - onehot(targets)) * scale, scale a one-element fp32 tensor on the device."""
+    _ce_check(logits, targets)
+    _dev(lse, scale)
+    if scale.dtype != torch.float32 or scale.numel() != 1 or lse.dtype != torch.float32 or not lse.is_contiguous():
+        raise RuntimeError("cross_entropy_bwd: lse must be contiguous fp32 [rows], scale one fp32 element")
+    rows, vocab = logits.shape
+    # same row pitch as the logits (a view into a padded buffer keeps its 16-byte-aligned rows)
+    out = logits if inplace else torch.empty_strided(logits.shape, logits.stride(), dtype=logits.dtype, device=logits.device)
+    check(_lib.lib().pico_cross_entropy_bwd(_ptr(logits), _ptr(targets), _ptr(lse), _ptr(scale), _ptr(out), rows, vocab,
+                                            logits.stride(0) if rows else vocab, out.stride(0) if rows else vocab,
+                                            ignore_index, _dt(logits, "logits"), _stream()))
+    return out

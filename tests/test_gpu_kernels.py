@@ -471,3 +471,27 @@ def test_fused_adamw_trains_like_torch_adamw_on_master_weights(device):
         assert maxabs(mine, r.detach()) <= 1e-5
         assert torch.equal(p.detach().cpu(), mine.to(torch.bfloat16).cpu())
         assert maxabs(p.detach().float(), r.detach()) <= 2 ** -8 * r.detach().abs().max().item()
+
+
+@pytest.mark.parametrize("rows,vocab,dtype", [(64, 49152, torch.bfloat16), (33, 1000, torch.bfloat16), (17, 515, torch.float32)])
+def test_cross_entropy_against_oracle(ops, device, rows, vocab, dtype):
+    """pico_cross_entropy_fwd / _bwd through the autograd function against the oracle: loss and lse to fp32 accuracy on
+    the same (rounded) logits, dlogits to the rounding of their dtype; ignored rows give no loss and no gradient."""
+    from oracle import layers as OL
+    from picotron_amd.functional import cross_entropy
+    g = torch.Generator().manual_seed(21)
+    x = (torch.randn(rows, vocab, generator=g) * 4).to(dtype)
+    t = torch.randint(0, vocab, (rows,), generator=g)
+    t[1] = -100
+    pitch = (vocab + 7) // 8 * 8   # rows start 16-byte aligned; the kernel's tail path covers vocab % vector != 0
+    xd = torch.zeros(rows, pitch, dtype=dtype, device=device)[:, :vocab].copy_(x.to(device)).requires_grad_()
+    loss = cross_entropy(xd, t.to(device))
+    (loss * 0.5).backward()
+    want, want_lse = OL.cross_entropy(x, t)
+    assert abs(loss.item() - want.item()) <= 2e-5 * max(1.0, abs(want.item()))
+    _, lse = ops.cross_entropy_fwd(xd.detach(), t.to(device))
+    assert maxabs(lse, want_lse) <= 2e-5 * want_lse.abs().max().item()
+    gw = OL.cross_entropy_backward(x, t, 0.5)
+    tol = 2 ** -8 if dtype == torch.bfloat16 else 1e-6
+    assert maxabs(xd.grad, gw) <= tol * gw.abs().max().item() + 1e-9
+    assert xd.grad[1].abs().max().item() == 0.0

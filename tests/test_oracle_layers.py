@@ -159,3 +159,21 @@ def test_adamw_step_matches_torch_adamw():
             assert (p - ref.detach()).abs().max().item() <= tol * max(1.0, p.abs().max().item())
         st = opt.state[ref]
         assert (m - st["exp_avg"]).abs().max().item() <= tol and (v - st["exp_avg_sq"]).abs().max().item() <= tol
+
+
+def test_cross_entropy_matches_torch():
+    """oracle.layers.cross_entropy / _backward against F.cross_entropy (the routine train.py:49 calls) and autograd,
+    with ignored rows."""
+    import torch.nn.functional as F
+    from oracle import layers as OL
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(37, 101, generator=g, dtype=torch.float64) * 3).requires_grad_()
+    t = torch.randint(0, 101, (37,), generator=g)
+    t[3] = -100
+    t[20] = -100
+    want = F.cross_entropy(x, t, reduction="mean")
+    got, lse = OL.cross_entropy(x.detach(), t)
+    assert abs(got.item() - want.item()) <= 1e-6
+    assert (lse - torch.logsumexp(x.detach(), -1)).abs().max().item() <= 1e-6
+    (gx,) = torch.autograd.grad(want * 0.7, x)
+    assert (OL.cross_entropy_backward(x.detach(), t, 0.7) - gx).abs().max().item() <= 1e-6
