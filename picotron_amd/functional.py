@@ -85,7 +85,7 @@ class FlashAttnFunc(torch.autograd.Function):
         # delta = sum_d dout * out is computed inside the call; gradients come back in the dtype and memory layout of
         # their inputs: no accumulation buffer, no cast pass
         dq, dk, dv = ops.attn_bwd(dout, q, k, v, lse, None, ctx.sm_scale, ctx.causal, 0, dq_dtype=q.dtype, dq_like=q,
-                                  dkv_dtype=k.dtype, out=out)
+                                  dkv_dtype=k.dtype, out=out, dkv_like=k if k.stride() == v.stride() else None)
         return dq, dk, dv, None, None
 
 
@@ -112,3 +112,85 @@ class CrossEntropyFunc(torch.autograd.Function):
 def cross_entropy(logits, targets, ignore_index: int = -100):
     """Drop-in for ``F.cross_entropy(logits, targets, reduction='mean')`` on 2-D logits."""
     return CrossEntropyFunc.apply(logits, targets, ignore_index)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Fused projections.  The reference's q_proj / k_proj / v_proj (and gate_proj / up_proj) read the same activation;
+# their weights are kept as separate Parameters but laid out back to back in one buffer, so one GEMM produces all
+# outputs, one GEMM all weight gradients and one GEMM the (already summed) input gradient.  The pieces below hand
+# strided views of those fused buffers to the kernels, which take row pitches / element strides as they are, and
+# write the pieces of the fused gradient in place: no concatenation, split or layout copy on either pass.
+
+class FusedLinearFunc(torch.autograd.Function):
+    """y = x @ w_fused^T where w_fused is the buffer that the Parameters `parts` (rows of it, in order) alias."""
+
+    @staticmethod
+    def forward(ctx, x, w_fused, *parts):
+        ctx.save_for_backward(x, w_fused)
+        ctx.sizes = [p.size(0) for p in parts]
+        return torch.nn.functional.linear(x, w_fused)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        dy2 = dy.reshape(-1, dy.size(-1))
+        dx = (dy2 @ w).view(x.shape)
+        dw = dy2.t() @ x.reshape(-1, x.size(-1))
+        return (dx, None) + tuple(dw.split(ctx.sizes, dim=0))
+
+
+class QKVAttentionFunc(torch.autograd.Function):
+    """RoPE on the q and k parts of a fused [B,S,(Hq+2Hkv)*D] projection, then causal / dense attention (one chunk);
+    returns [B,S,Hq*D].  The backward writes dq, dk, dv straight into the matching columns of one [B,S,(Hq+2Hkv)*D]
+    buffer and un-rotates dq and dk there in place."""
+
+    @staticmethod
+    def forward(ctx, qkv, cos, sin, n_heads, n_kv_heads, head_dim, causal):
+        B, S, _ = qkv.shape
+        nq, nkv = n_heads * head_dim, n_kv_heads * head_dim
+        q = qkv[..., :nq].view(B, S, n_heads, head_dim).transpose(1, 2)
+        k = qkv[..., nq:nq + nkv].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
+        v = qkv[..., nq + nkv:].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
+        # rotated copies in [B,S,H,D] memory (the projection output itself stays untouched: v is used as it lies)
+        q = ops.rope(q, cos, sin, 0, out=ops.empty_bshd(B, n_heads, S, head_dim, qkv.dtype, qkv.device))
+        k = ops.rope(k, cos, sin, 0, out=ops.empty_bshd(B, n_kv_heads, S, head_dim, qkv.dtype, qkv.device))
+        sm_scale = 1.0 / (head_dim ** 0.5)
+        out, lse = ops.attn_fwd(q, k, v, sm_scale, causal, 0, out_dtype=qkv.dtype, bshd_out=True)
+        ctx.save_for_backward(q, k, v, out, lse, cos, sin)
+        ctx.meta = (n_heads, n_kv_heads, head_dim, causal, sm_scale)
+        return out.transpose(1, 2).reshape(B, S, nq)
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, cos, sin = ctx.saved_tensors
+        n_heads, n_kv_heads, head_dim, causal, sm_scale = ctx.meta
+        B, S = q.size(0), q.size(2)
+        nq, nkv = n_heads * head_dim, n_kv_heads * head_dim
+        dqkv = torch.empty(B, S, nq + 2 * nkv, dtype=q.dtype, device=q.device)
+        dq = dqkv[..., :nq].view(B, S, n_heads, head_dim).transpose(1, 2)
+        dk = dqkv[..., nq:nq + nkv].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
+        dv = dqkv[..., nq + nkv:].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
+        do = dout.view(B, S, n_heads, head_dim).transpose(1, 2)
+        ops.attn_bwd(do, q, k, v, lse, None, sm_scale, causal, 0, dq, dk, dv, out=out)
+        ops.rope(dq, cos, sin, 0, inverse=True, out=dq)
+        ops.rope(dk, cos, sin, 0, inverse=True, out=dk)
+        return dqkv, None, None, None, None, None, None
+
+
+class SwiGLUFusedFunc(torch.autograd.Function):
+    """silu(gate) * up where gate and up are the two halves of one [..., 2I] projection output; the backward writes
+    dgate and dup into the halves of one [..., 2I] buffer."""
+
+    @staticmethod
+    def forward(ctx, gate_up):
+        ctx.save_for_backward(gate_up)
+        half = gate_up.size(-1) // 2
+        return ops.swiglu_fwd(gate_up[..., :half], gate_up[..., half:])
+
+    @staticmethod
+    def backward(ctx, dy):
+        (gate_up,) = ctx.saved_tensors
+        half = gate_up.size(-1) // 2
+        d = torch.empty_like(gate_up)
+        ops.swiglu_bwd(dy, gate_up[..., :half], gate_up[..., half:], out=(d[..., :half], d[..., half:]))
+        return d

@@ -34,7 +34,8 @@ import torch.nn.functional as F
 
 import picotron_amd.process_group_manager as pgm
 from picotron_amd.context_parallel import context_parallel
-from picotron_amd.functional import FlashAttnFunc, RMSNormFunc, RMSNormResidualFunc, RotaryFunc, SwiGLUFunc
+from picotron_amd.functional import (FlashAttnFunc, FusedLinearFunc, QKVAttentionFunc, RMSNormFunc, RMSNormResidualFunc,
+                                     RotaryFunc, SwiGLUFunc, SwiGLUFusedFunc)
 
 
 def apply_rotary_pos_emb(x, cos, sin):
@@ -102,6 +103,34 @@ class LlamaRMSNorm(nn.Module):
         return RMSNormFunc.apply(hidden_states, self.weight, self.variance_epsilon, True)
 
 
+def _fused_projections() -> bool:
+    """One GEMM for q/k/v and one for gate/up (default); PICO_FUSED_PROJ=0 keeps the reference's separate GEMMs."""
+    return os.getenv("PICO_FUSED_PROJ", "1") != "0"
+
+
+def _fused_weight(owner, name, linears):
+    """The [sum(out_i), in] buffer that the weights of `linears` alias, row block by row block.  Built on first use
+    and rebuilt whenever the Parameters were moved or cast since (``model.to(...)`` gives them fresh storage); the
+    Parameters stay separate leaves with their own names, gradients and optimizer state."""
+    ws = [m.weight for m in linears]
+    buf = owner.__dict__.get(name)
+    ok = buf is not None and buf.dtype == ws[0].dtype and buf.device == ws[0].device
+    if ok:
+        ptr = buf.data_ptr()
+        for w in ws:
+            ok = ok and w.data_ptr() == ptr and w.is_contiguous()
+            ptr += w.numel() * w.element_size()
+    if not ok:
+        with torch.no_grad():
+            buf = torch.cat([w.detach() for w in ws], dim=0).contiguous()
+            row = 0
+            for w in ws:
+                w.data = buf[row:row + w.size(0)]
+                row += w.size(0)
+        owner.__dict__[name] = buf
+    return buf
+
+
 def _fan_in_uniform_(tensor):
     bound = math.sqrt(1 / tensor.size(1))
     torch.nn.init.uniform_(tensor, -bound, bound)
@@ -133,6 +162,13 @@ class Attention(nn.Module):
 
     def forward(self, x, cos, sin, attention_mask=None, position_ids=None):
         batch_size, seq_length, _ = x.size()
+        context = os.getenv("CONTEXT_PARALLEL", "0") == "1"
+        if _fused_projections() and not context and cos.size(0) >= seq_length:
+            # one GEMM for q, k and v; RoPE, attention and their backward work on strided views of the fused buffers
+            w = _fused_weight(self, "_qkv_weight", (self.q_proj, self.k_proj, self.v_proj))
+            qkv = FusedLinearFunc.apply(x, w, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
+            out = QKVAttentionFunc.apply(qkv, cos, sin, self.num_local_heads, self.num_local_kv_heads, self.head_dim, True)
+            return self.out_proj(out)
         # [B,S,H*D] -> [B,H,S,D] views over [B,S,H,D] memory; the kernels take the strides as they are
         q = self.q_proj(x).view(batch_size, seq_length, self.num_local_heads, self.head_dim).transpose(1, 2)
         k = self.k_proj(x).view(batch_size, seq_length, self.num_local_kv_heads, self.head_dim).transpose(1, 2)
@@ -166,6 +202,10 @@ class MLP(nn.Module):
             _fan_in_uniform_(proj.weight)
 
     def forward(self, x):
+        if _fused_projections():
+            w = _fused_weight(self, "_gate_up_weight", (self.gate_proj, self.up_proj))
+            gate_up = FusedLinearFunc.apply(x, w, self.gate_proj.weight, self.up_proj.weight)
+            return self.down_proj(SwiGLUFusedFunc.apply(gate_up))
         return self.down_proj(SwiGLUFunc.apply(self.gate_proj(x), self.up_proj(x)))
 
 

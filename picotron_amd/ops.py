@@ -111,6 +111,8 @@ def _dense(t: torch.Tensor) -> bool:
 
 # ------------------------------------------------------------------------------- SwiGLU
 def _as_2d(t: torch.Tensor) -> torch.Tensor:
+    """[..., C] -> [rows, C] without a copy when the leading dims collapse to one row pitch (a column slice of a
+    contiguous buffer does); a copy otherwise."""
     if t.stride(-1) != 1:
         t = t.contiguous()
     if t.dim() == 2:
@@ -118,7 +120,12 @@ def _as_2d(t: torch.Tensor) -> torch.Tensor:
     try:
         return t.view(-1, t.size(-1))
     except RuntimeError:
-        return t.contiguous().view(-1, t.size(-1))
+        pass
+    # leading dims with a common pitch: stride[i] == stride[i+1] * size[i+1]
+    if all(t.stride(i) == t.stride(i + 1) * t.size(i + 1) for i in range(t.dim() - 2)):
+        rows = t.numel() // t.size(-1)
+        return t.as_strided((rows, t.size(-1)), (t.stride(-2), 1))
+    return t.contiguous().view(-1, t.size(-1))
 
 
 def swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
@@ -133,12 +140,20 @@ def swiglu_fwd(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     return y
 
 
-def swiglu_bwd(dy: torch.Tensor, gate: torch.Tensor, up: torch.Tensor):
+def swiglu_bwd(dy: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, out=None):
+    """(dgate, dup); `out` = (dgate, dup) buffers to write into (e.g. the two halves of one fused gradient)."""
     _dev(dy, gate, up)
     g2, u2, d2 = _as_2d(gate), _as_2d(up), _as_2d(dy.to(gate.dtype))
-    dg = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
-    du = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
-    dg2, du2 = dg.view(-1, dg.size(-1)), du.view(-1, du.size(-1))
+    if out is None:
+        dg = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+        du = torch.empty(gate.shape, dtype=gate.dtype, device=gate.device)
+    else:
+        dg, du = out
+        if dg.shape != gate.shape or du.shape != gate.shape or dg.dtype != gate.dtype or du.dtype != gate.dtype:
+            raise RuntimeError("swiglu_bwd: out buffers must match gate in shape and dtype")
+    dg2, du2 = _as_2d(dg), _as_2d(du)
+    if dg2.data_ptr() != dg.data_ptr() or du2.data_ptr() != du.data_ptr():
+        raise RuntimeError("swiglu_bwd: out buffers need a unit last stride and one row pitch")
     check(_lib.lib().pico_swiglu_bwd(_ptr(d2), _ptr(g2), _ptr(u2), _ptr(dg2), _ptr(du2), g2.size(0), g2.size(1),
                                      d2.stride(0), g2.stride(0), u2.stride(0), dg2.stride(0), du2.stride(0),
                                      _dt(gate, "swiglu_bwd"), _stream()))
@@ -246,12 +261,13 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
              dq_accumulate: bool = False, dkv_accumulate: bool = False, dq_dtype=torch.float32,
              dkv_dtype=torch.float32, dq_like: Optional[torch.Tensor] = None, want_dq: bool = True,
              want_dkv: bool = True, side_stream: Optional["torch.cuda.Stream"] = None,
-             out: Optional[torch.Tensor] = None):
+             out: Optional[torch.Tensor] = None, dkv_like: Optional[torch.Tensor] = None):
     """Gradients of one attention block; returns (dq [B,Hq,Sq,D], dk, dv [B,Hkv,Sk,D]).
 
     Buffers that are passed in are written in place (fp32 ones can be accumulated into: the running dq of a
     rank and the travelling dk / dv of the ring); missing ones are allocated in the requested dtype, dq with
-    the strides of `dq_like` if given.  want_dq / want_dkv = False skips that gradient (and its kernel).
+    the strides of `dq_like` if given, dk / dv with the strides of `dkv_like` (so that a gradient for a [B,H,S,D] view
+    of [B,S,H,D] memory needs no layout copy on its way back).  want_dq / want_dkv = False skips that gradient.
     With `out` (the forward output) `delta` may be None or a buffer to fill: the row sums delta = sum_d dout * out are
     then computed inside the call (by the dQ kernel itself when out is bf16 and dq is wanted), as in the reference's
     ring_attention_backward, instead of by a separate attn_bwd_preprocess.
@@ -285,8 +301,12 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
     if (dk is None or dv is None) and want_dkv:
         if dkv_accumulate:
             raise RuntimeError("attn_bwd: dkv_accumulate=True needs existing dk / dv")
-        dk = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
-        dv = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
+        if dkv_like is not None and _dense(dkv_like) and dkv_like.stride(-1) == 1 and dkv_like.shape == k.shape:
+            dk = torch.empty_strided(k.shape, dkv_like.stride(), dtype=dkv_dtype, device=q.device)
+            dv = torch.empty_strided(k.shape, dkv_like.stride(), dtype=dkv_dtype, device=q.device)
+        else:
+            dk = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
+            dv = torch.empty(B, Hkv, Sk, D, dtype=dkv_dtype, device=q.device)
     if not want_dq:
         dq = None
     if not want_dkv:

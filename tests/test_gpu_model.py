@@ -217,3 +217,35 @@ def test_model_cp4_virtual_ranks_equals_cp1(pgm1, device):
     mgr.cp_ring.reset()
     pgm.setup_process_group_manager(1, 1, 1, 1)
     os.environ["CONTEXT_PARALLEL"] = "0"
+
+
+def test_fused_projections_match_separate_projections(pgm1, device):
+    """PICO_FUSED_PROJ: one GEMM for q/k/v (RoPE + attention on strided views, gradients written into one fused buffer)
+    and one for gate/up must give the separate-GEMM path's loss and parameter gradients; the Parameters keep their
+    names, and survive a cast (which gives them fresh storage) by being re-fused."""
+    from picotron_amd.functional import cross_entropy
+    from picotron_amd.model import Llama
+    cfg = OM.LlamaShape(256, 4, 2, 512, 1024, 2, 128)
+    ids, tgt = OM.synthetic_batch(cfg.vocab_size, 2, 128, seed=3)
+    ids, tgt = ids.to(device), tgt.to(device)
+    grads = {}
+    try:
+        for mode in ("0", "1"):
+            os.environ["PICO_FUSED_PROJ"] = mode
+            torch.manual_seed(0)
+            m = Llama(cfg).to(device).to(torch.bfloat16)
+            if mode == "1":
+                m(ids)                      # fuse, then cast there and back (exact): fresh storage, must be re-fused
+                m = m.to(torch.float32).to(torch.bfloat16)
+            loss = cross_entropy(m(ids).view(-1, cfg.vocab_size), tgt.reshape(-1))
+            loss.backward()
+            grads[mode] = (loss.item(), {n: p.grad.float().cpu() for n, p in m.named_parameters()})
+            if mode == "1":
+                att = m.decoder_layers[0].attention
+                assert att.k_proj.weight.data_ptr() == att.q_proj.weight.data_ptr() + att.q_proj.weight.numel() * 2
+    finally:
+        os.environ.pop("PICO_FUSED_PROJ", None)
+    assert set(grads["0"][1]) == set(grads["1"][1])
+    assert abs(grads["0"][0] - grads["1"][0]) <= 2e-3
+    for n, g0 in grads["0"][1].items():
+        assert rel_l2(grads["1"][1][n], g0) <= 2e-2, n
