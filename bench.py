@@ -279,7 +279,7 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3):
     # the bf16 parameter (picotron_amd.optim.FusedAdamW over pico_adamw)
     from picotron_amd.functional import cross_entropy
     from picotron_amd.optim import FusedAdamW
-    opt = FusedAdamW(model.parameters(), lr=3e-4)
+    opt = FusedAdamW(model.parameters(), lr=3e-4, overlap_with_backward=os.getenv("PICO_BENCH_OVERLAP", "0") == "1")
     ids, tgt = synthetic_batch(cfg.vocab_size, mbs, seq, seed=0)
     ids, tgt = ids.cuda(), tgt.cuda()
 

@@ -495,3 +495,24 @@ def test_cross_entropy_against_oracle(ops, device, rows, vocab, dtype):
     tol = 2 ** -8 if dtype == torch.bfloat16 else 1e-6
     assert maxabs(xd.grad, gw) <= tol * gw.abs().max().item() + 1e-9
     assert xd.grad[1].abs().max().item() == 0.0
+
+
+def test_fused_adamw_overlapped_with_backward_gives_the_same_update(device):
+    """overlap_with_backward updates each parameter from a hook on a second stream; same numbers as step()."""
+    from picotron_amd.optim import FusedAdamW
+    results = []
+    for overlap in (False, True):
+        torch.manual_seed(5)
+        lin1 = torch.nn.Linear(64, 48, bias=False).to(device).to(torch.bfloat16)
+        lin2 = torch.nn.Linear(48, 8, bias=False).to(device).to(torch.bfloat16)
+        params = list(lin1.parameters()) + list(lin2.parameters())
+        opt = FusedAdamW(params, lr=1e-2, overlap_with_backward=overlap)
+        x = torch.randn(16, 64, device=device).to(torch.bfloat16)
+        for _ in range(3):
+            opt.zero_grad()
+            lin2(torch.tanh(lin1(x))).float().square().mean().backward()
+            opt.step()
+        torch.cuda.synchronize()
+        results.append([p.detach().float().cpu() for p in params] + [opt.master.cpu()])
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
