@@ -253,6 +253,21 @@ def bandwidth_extras(torch, ops, iters=50):
         lambda g_, u: ops.swiglu_fwd(g_, u), 3 * T * I * 2, 4)
     run("swiglu_bwd", lambda: tuple(torch.randn(T, I, device=dev).to(bf) for _ in range(3)),
         lambda dy, g_, u: ops.swiglu_bwd(dy, g_, u), 5 * T * I * 2, 3)
+    # cross-entropy over the 49152-entry vocabulary of the step: forward reads the logits once, backward reads them
+    # again and writes dlogits
+    Vc = 49152
+    tg = torch.randint(0, Vc, (T,), device=dev)
+    one = torch.ones(1, device=dev)
+    run("cross_entropy_fwd", lambda: (torch.randn(T, Vc, device=dev).to(bf),),
+        lambda lg: ops.cross_entropy_fwd(lg, tg), T * Vc * 2, 2)
+    lse_c = ops.cross_entropy_fwd(torch.randn(T, Vc, device=dev).to(bf), tg)[1]
+    run("cross_entropy_bwd", lambda: (torch.randn(T, Vc, device=dev).to(bf),),
+        lambda lg: ops.cross_entropy_bwd(lg, tg, lse_c, one), 2 * T * Vc * 2, 2)
+    # AdamW with fp32 master weights and moments on 64 Mi bf16 parameters: 28 bytes per parameter
+    n = 64 * 1024 * 1024
+    run("adamw", lambda: (torch.zeros(n, device=dev, dtype=bf), torch.randn(n, device=dev), torch.randn(n, device=dev).to(bf),
+                          torch.zeros(n, device=dev), torch.zeros(n, device=dev)),
+        lambda p_, m_, g_, ea, eas: ops.adamw_(p_, m_, g_, ea, eas, 1, 1e-3), 28 * n, 1)
     return res
 
 
