@@ -219,6 +219,14 @@ int pico_cross_entropy_bwd(const void* logits, const int64_t* targets, const flo
 int pico_adamw(void* param_lp, float* master, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
                int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step,
                float grad_scale, void* stream);
+/* The same step with the state held as the reference holds it for a bf16 model (train.py:209 builds AdamW on the
+ * bf16 parameters, so torch keeps exp_avg and exp_avg_sq in bf16 and updates the bf16 parameter itself): param,
+ * exp_avg, exp_avg_sq are [n] of `dtype` (PICO_BF16), updated in place; the arithmetic is fp32 and each state is
+ * rounded once per step (what torch's fused AdamW does; its default for-each path rounds after every operation).
+ */
+int pico_adamw_lp(void* param, const void* grad, int grad_dtype, void* exp_avg, void* exp_avg_sq, int64_t n, int dtype,
+                  float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step, float grad_scale,
+                  void* stream);
 
 #ifdef __cplusplus
 }

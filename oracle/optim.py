@@ -3,7 +3,13 @@
 torch applies it.  Test infrastructure only.  The reference keeps the AdamW state in the parameter dtype; the
 build under test keeps fp32 master weights and moments for bf16 parameters, which is what ``master_step`` states.
 
-Pinned by ``tests/test_oracle_layers.py`` against ``torch.optim.AdamW`` itself (a library routine) over several steps.
+``lp_step`` states the reference's own layout -- parameter and moments in the parameter dtype -- with fp32 arithmetic
+and one rounding per state, which is what torch's ``fused=True`` AdamW computes (its default for-each path rounds
+after every operation instead).
+
+Pinned by ``tests/test_oracle_layers.py`` against ``torch.optim.AdamW`` itself (a library routine) over several steps:
+``adamw_step`` against the default implementation on fp32 parameters, ``lp_step`` against ``fused=True`` on bf16
+parameters.
 """
 from __future__ import annotations
 
@@ -31,3 +37,10 @@ def master_step(master: torch.Tensor, grad_lp: torch.Tensor, m: torch.Tensor, v:
     new parameter (what the model computes with)."""
     p, m, v = adamw_step(master.float(), grad_lp.float(), m.float(), v.float(), step, lr, **kw)
     return p, m, v, p.to(lp_dtype)
+
+
+def lp_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor, step: int, lr: float, **kw):
+    """AdamW with parameter and both moments stored in p.dtype: fp32 arithmetic, each state rounded once."""
+    dt = p.dtype
+    p2, m2, v2 = adamw_step(p.float(), g.float(), m.float(), v.float(), step, lr, **kw)
+    return p2.to(dt), m2.to(dt), v2.to(dt)

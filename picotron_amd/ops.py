@@ -387,6 +387,24 @@ def adamw_(param_lp: Optional[torch.Tensor], master: torch.Tensor, grad: torch.T
                                 float(grad_scale), _stream()))
 
 
+def adamw_lp_(param: torch.Tensor, grad: torch.Tensor, exp_avg: torch.Tensor, exp_avg_sq: torch.Tensor, step: int,
+              lr: float, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8, weight_decay: float = 0.01,
+              grad_scale: float = 1.0) -> None:
+    """In-place AdamW step on a bf16 parameter with bf16 moments (the state torch.optim.AdamW holds for a bf16
+    model); fp32 arithmetic, one rounding per state.  `step` counts from 1."""
+    _dev(param, grad, exp_avg, exp_avg_sq)
+    n = param.numel()
+    for t, what in ((param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != n:
+            raise RuntimeError(f"adamw_lp_: {what} must be a contiguous bf16 tensor of {n} elements")
+    if grad.numel() != n:
+        raise RuntimeError("adamw_lp_: grad has the wrong number of elements")
+    grad = grad.contiguous()
+    check(_lib.lib().pico_adamw_lp(_ptr(param), _ptr(grad), _dt(grad, "grad"), _ptr(exp_avg), _ptr(exp_avg_sq), n,
+                                   _dt(param, "param"), float(lr), float(beta1), float(beta2), float(eps),
+                                   float(weight_decay), int(step), float(grad_scale), _stream()))
+
+
 def _ce_check(logits: torch.Tensor, targets: torch.Tensor):
     _dev(logits, targets)
     if logits.dim() != 2 or logits.stride(1) != 1:

@@ -1,9 +1,13 @@
-"""AdamW for bf16 parameters with fp32 master weights and moments, one fused HIP pass per parameter tensor.
+"""AdamW for the model's parameters, one fused HIP pass per parameter tensor.
 
 The reference builds ``torch.optim.AdamW(model.parameters(), lr)`` (``train.py:204-209``; its ``fused`` switch is
-dead code) and so keeps the optimizer state in the parameter dtype.  Here the state is fp32: a master copy of every
-parameter plus both moments, laid out in three flat buffers, and ``step()`` reads each bf16 gradient once and rewrites
-the bf16 parameter from the updated master weight in the same kernel (``pico_adamw``) -- no cast passes."""
+dead code) on the bf16 model and so keeps the optimizer state in the parameter dtype.  Two layouts are offered:
+
+``master_weights=True`` (default)  fp32 state: a master copy of every parameter plus both moments in three flat
+    buffers; ``step()`` reads each bf16 gradient once and rewrites the bf16 parameter from the updated master weight
+    in the same kernel (``pico_adamw``) -- no cast passes.  28 bytes of HBM traffic per parameter.
+``master_weights=False``  the reference's layout: the bf16 parameter is updated in place and both moments are bf16
+    (``pico_adamw_lp``); fp32 arithmetic inside the kernel, one rounding per state.  14 bytes per parameter."""
 from __future__ import annotations
 
 from typing import Iterable
@@ -15,7 +19,7 @@ from . import ops
 
 class FusedAdamW:
     def __init__(self, params: Iterable[torch.nn.Parameter], lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
-                 weight_decay: float = 1e-2, overlap_with_backward: bool = False):
+                 weight_decay: float = 1e-2, overlap_with_backward: bool = False, master_weights: bool = True):
         self.params = [p for p in params if p.requires_grad]
         if not self.params:
             raise ValueError("FusedAdamW: no parameters")
@@ -30,11 +34,19 @@ class FusedAdamW:
         for p in self.params:
             self.offsets.append(total)
             total += (p.numel() + 7) // 8 * 8
-        self.master = torch.zeros(total, dtype=torch.float32, device=dev)
-        self.exp_avg = torch.zeros(total, dtype=torch.float32, device=dev)
-        self.exp_avg_sq = torch.zeros(total, dtype=torch.float32, device=dev)
-        for p, off in zip(self.params, self.offsets):
-            self.master[off:off + p.numel()].copy_(p.detach().reshape(-1))
+        self.master_weights = master_weights
+        if master_weights:
+            state_dtype = torch.float32
+            self.master = torch.zeros(total, dtype=torch.float32, device=dev)
+            for p, off in zip(self.params, self.offsets):
+                self.master[off:off + p.numel()].copy_(p.detach().reshape(-1))
+        else:
+            state_dtype = self.params[0].dtype
+            if any(p.dtype != state_dtype for p in self.params):
+                raise RuntimeError("FusedAdamW(master_weights=False): all parameters must share one dtype")
+            self.master = None
+        self.exp_avg = torch.zeros(total, dtype=state_dtype, device=dev)
+        self.exp_avg_sq = torch.zeros(total, dtype=state_dtype, device=dev)
         # Optional: update each parameter on a second stream as soon as the backward pass has produced its gradient.
         # The update is a pure HBM stream and the rest of the backward is GEMM-bound, so the two can overlap (measured:
         # +1 % tokens/s on the SmolLM-1.7B-shaped step, so it is off by default); a weight is read only by its own
@@ -47,19 +59,28 @@ class FusedAdamW:
             for i, p in enumerate(self.params):
                 p.register_post_accumulate_grad_hook(lambda p_, i_=i: self._on_grad(i_, p_))
 
+    def _update(self, p, off, g, grad_scale):
+        n = p.numel()
+        m, v = self.exp_avg[off:off + n], self.exp_avg_sq[off:off + n]
+        hyper = (self.step_count, self.lr, self.betas[0], self.betas[1], self.eps, self.weight_decay, grad_scale)
+        if self.master_weights:
+            ops.adamw_(p if p.dtype == torch.bfloat16 else None, self.master[off:off + n], g, m, v, *hyper)
+            if p.dtype == torch.float32:
+                p.copy_(self.master[off:off + n].view_as(p))
+        elif p.dtype == torch.bfloat16:
+            ops.adamw_lp_(p.view(-1), g, m, v, *hyper)
+        else:
+            ops.adamw_(None, p.view(-1), g, m, v, *hyper)
+
     @torch.no_grad()
     def _on_grad(self, i, p):
         if not self._open or p.grad is None:
             return
         cur = torch.cuda.current_stream()
         self.side.wait_stream(cur)
-        off, n, g = self.offsets[i], p.numel(), p.grad
+        off, g = self.offsets[i], p.grad
         with torch.cuda.stream(self.side):
-            ops.adamw_(p if p.dtype == torch.bfloat16 else None, self.master[off:off + n], g,
-                       self.exp_avg[off:off + n], self.exp_avg_sq[off:off + n], self.step_count, self.lr, self.betas[0],
-                       self.betas[1], self.eps, self.weight_decay, 1.0)
-            if p.dtype == torch.float32:
-                p.copy_(self.master[off:off + n].view_as(p))
+            self._update(p, off, g, 1.0)
         g.record_stream(self.side)   # its memory must not be handed out again before the side stream has read it
         p.grad = None
 
@@ -85,9 +106,4 @@ class FusedAdamW:
         for p, off in zip(self.params, self.offsets):
             if p.grad is None:
                 continue
-            n = p.numel()
-            ops.adamw_(p if p.dtype == torch.bfloat16 else None, self.master[off:off + n], p.grad,
-                       self.exp_avg[off:off + n], self.exp_avg_sq[off:off + n], self.step_count, self.lr, self.betas[0],
-                       self.betas[1], self.eps, self.weight_decay, grad_scale)
-            if p.dtype == torch.float32:
-                p.copy_(self.master[off:off + n].view_as(p))
+            self._update(p, off, p.grad, grad_scale)

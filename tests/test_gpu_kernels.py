@@ -452,6 +452,52 @@ def test_adamw_kernel_against_oracle(ops, device, n, grad_dtype):
         assert torch.equal(d_p.cpu(), d_master.cpu().to(torch.bfloat16))
 
 
+@pytest.mark.parametrize("n,grad_dtype", [(8 * 1024 + 3, torch.bfloat16), (4096, torch.float32), (5, torch.bfloat16)])
+def test_adamw_lp_kernel_against_oracle(ops, device, n, grad_dtype):
+    """pico_adamw_lp (bf16 parameter and moments updated in place) over four steps against oracle.optim.lp_step fed the
+    kernel's own previous state: both compute in fp32 and round once, so almost every element is identical and the rest
+    are one bf16 rounding step apart (the compiler may contract a multiply-add that the oracle rounds twice)."""
+    from oracle import optim as OO
+    g = torch.Generator().manual_seed(13)
+    p = torch.randn(n, generator=g).bfloat16()
+    d_p, d_m, d_v = p.to(device), torch.zeros(n, dtype=torch.bfloat16, device=device), torch.zeros(n, dtype=torch.bfloat16, device=device)
+    for step in range(1, 5):
+        grad = (torch.randn(n, generator=g) * 0.05 * step).to(grad_dtype)
+        want = OO.lp_step(d_p.cpu(), grad, d_m.cpu(), d_v.cpu(), step, 2e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
+        ops.adamw_lp_(d_p, grad.to(device), d_m, d_v, step, 2e-3, 0.9, 0.95, 1e-8, 0.1)
+        for got, w in zip((d_p, d_m, d_v), want):
+            diff = (got.cpu().float() - w.float()).abs()
+            assert (diff <= w.float().abs() * 2.0 ** -7 + w.float().abs().mean() * 2.0 ** -14).all()
+            assert (diff != 0).sum().item() <= max(1, 0.03 * n)
+
+
+def test_fused_adamw_without_master_weights_follows_torch_fused_adamw(device):
+    """FusedAdamW(master_weights=False) keeps the reference's state layout (train.py:209: AdamW on the bf16
+    parameters); torch.optim.AdamW(fused=True) on bf16 copies, fed the same gradients, computes the same way (fp32
+    arithmetic, one rounding per state), so parameters and moments agree to a rounding step after three steps."""
+    from picotron_amd.optim import FusedAdamW
+    torch.manual_seed(5)
+    ps = [torch.nn.Parameter(torch.randn(33, 20, device=device).to(torch.bfloat16)), torch.nn.Parameter(torch.randn(7, device=device).to(torch.bfloat16))]
+    ref = [torch.nn.Parameter(p.detach().clone()) for p in ps]
+    opt = FusedAdamW(ps, lr=1e-2, weight_decay=0.02, master_weights=False)
+    ropt = torch.optim.AdamW(ref, lr=1e-2, weight_decay=0.02, fused=True)
+    assert opt.master is None and opt.exp_avg.dtype == torch.bfloat16
+    for _ in range(3):
+        for p, r in zip(ps, ref):
+            p.grad = torch.randn_like(p)
+            r.grad = p.grad.clone()
+        opt.step()
+        ropt.step()
+    for p, r, off in zip(ps, ref, opt.offsets):
+        n = p.numel()
+        st = ropt.state[r]
+        for got, w in ((p.detach(), r.detach()), (opt.exp_avg[off:off + n].view_as(p), st["exp_avg"]),
+                       (opt.exp_avg_sq[off:off + n].view_as(p), st["exp_avg_sq"])):
+            diff = (got.float() - w.float()).abs()
+            assert (diff <= w.float().abs() * 2.0 ** -7 + w.float().abs().mean() * 2.0 ** -7).all()
+            assert (diff != 0).sum().item() <= max(1, 0.05 * n)
+
+
 def test_fused_adamw_trains_like_torch_adamw_on_master_weights(device):
     """picotron_amd.optim.FusedAdamW on bf16 parameters follows torch.optim.AdamW run on fp32 copies fed the same
     bf16 gradients."""

@@ -161,6 +161,32 @@ def test_adamw_step_matches_torch_adamw():
         assert (m - st["exp_avg"]).abs().max().item() <= tol and (v - st["exp_avg_sq"]).abs().max().item() <= tol
 
 
+def test_adamw_lp_step_matches_torch_fused_adamw():
+    """oracle.optim.lp_step (bf16 parameter and moments, fp32 arithmetic, one rounding per state) against
+    torch.optim.AdamW(fused=True) on a bf16 parameter: after five steps every state is within one bf16 ulp and
+    almost all are identical (the two may order a multiplication differently inside fp32)."""
+    from oracle import optim as OO
+    g = torch.Generator().manual_seed(11)
+    p0 = torch.randn(4099, generator=g).bfloat16()
+    ref = torch.nn.Parameter(p0.clone())
+    try:
+        opt = torch.optim.AdamW([ref], lr=3e-3, betas=(0.85, 0.97), eps=1e-7, weight_decay=0.05, fused=True)
+    except RuntimeError as e:   # a torch build without the fused CPU kernel
+        pytest.skip(f"torch has no fused AdamW on the CPU: {e}")
+    p, m, v = p0.clone(), torch.zeros_like(p0), torch.zeros_like(p0)
+    for step in range(1, 6):
+        grad = (torch.randn(4099, generator=g) * (0.1 * step)).bfloat16()
+        ref.grad = grad.clone()
+        opt.step()
+        p, m, v = OO.lp_step(p, grad, m, v, step, 3e-3, beta1=0.85, beta2=0.97, eps=1e-7, weight_decay=0.05)
+    st = opt.state[ref]
+    for got, want in ((p, ref.detach()), (m, st["exp_avg"]), (v, st["exp_avg_sq"])):
+        assert got.dtype == want.dtype == torch.bfloat16
+        diff = (got.float() - want.float()).abs()
+        assert (diff <= want.float().abs() * 2.0 ** -7 + want.float().abs().mean() * 2.0 ** -7).all()
+        assert (diff == 0).float().mean().item() >= 0.98
+
+
 def test_cross_entropy_matches_torch():
     """oracle.layers.cross_entropy / _backward against F.cross_entropy (the routine train.py:49 calls) and autograd,
     with ignored rows."""
