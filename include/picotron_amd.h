@@ -67,11 +67,14 @@ int64_t pico_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t hidden);
 /* replaces: autograd of model.py:81-86 / the Triton backward of layer_norm_fn.
  * dx = rstd * (g - xhat * mean(g * xhat)),  g = dy * w,  xhat = x * rstd;  dweight = sum_rows dy * xhat.
  * x is the tensor that was normalised (after the residual add, if any).
- * dx: [rows, hidden] `dtype`; dweight: [hidden] fp32; workspace: device scratch of at least
- * pico_rmsnorm_bwd_workspace_bytes() bytes (contents undefined on entry and exit).
+ * dresidual: optional [rows, hidden] `dtype`, added to dx -- the gradient that reached the residual stream directly
+ *   when the forward fused the residual add (the dresidual input of layer_norm_fn's backward); dx may alias it.
+ * dx: [rows, hidden] `dtype` (may alias dy); dweight: [hidden] of dweight_dtype (PICO_F32 or PICO_BF16; summed in fp32
+ *   and rounded once); workspace: device scratch of at least pico_rmsnorm_bwd_workspace_bytes() bytes (contents
+ *   undefined on entry and exit).
  */
-int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
-                     void* dx, float* dweight, void* workspace, int64_t workspace_bytes,
+int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd, const void* dresidual,
+                     void* dx, void* dweight, int dweight_dtype, void* workspace, int64_t workspace_bytes,
                      int64_t rows, int64_t hidden, int dtype, void* stream);
 
 /* ------------------------------------------------------------------ RoPE
@@ -227,6 +230,18 @@ int pico_adamw(void* param_lp, float* master, const void* grad, int grad_dtype, 
 int pico_adamw_lp(void* param, const void* grad, int grad_dtype, void* exp_avg, void* exp_avg_sq, int64_t n, int dtype,
                   float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step, float grad_scale,
                   void* stream);
+/* The step for `count` tensors at once (what torch's for-each / fused AdamW does for the whole parameter list of
+ * train.py:209): host arrays of `count` device pointers and sizes; the library packs them into the arguments of as
+ * few launches as they fit (48 tensors each), so a model's ~200 parameter tensors cost 5 launches instead of 200.
+ * state_dtype PICO_F32: weights are the fp32 master weights and param_lps (the array or single entries may be NULL)
+ * receive their bf16 copies, as pico_adamw; PICO_BF16: weights are the bf16 parameters themselves and param_lps must
+ * be NULL, as pico_adamw_lp.  All gradients share grad_dtype.  Tensors of size 0 are skipped.  Every tensor is
+ * checked before the first launch: a rejected call has changed nothing.
+ */
+int pico_adamw_multi(int count, void* const* weights, void* const* param_lps, const void* const* grads,
+                     void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int state_dtype,
+                     int grad_dtype, float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step,
+                     float grad_scale, void* stream);
 
 #ifdef __cplusplus
 }

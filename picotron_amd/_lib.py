@@ -31,7 +31,7 @@ SIGNATURES = {
     "pico_last_error": (c_char_p, []),
     "pico_rmsnorm_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, c_float, c_int, c_int, _P]),
     "pico_rmsnorm_bwd_workspace_bytes": (_I64, [_I64, _I64]),
-    "pico_rmsnorm_bwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I64, _I64, _I64, c_int, _P]),
+    "pico_rmsnorm_bwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, _P, _I64, _I64, _I64, c_int, _P]),
     "pico_rope": (c_int, [_P, _P, _P, _P] + [_I64] * 4 + [_I64] * 6 + [_I64, _I64, c_int, c_int, c_int, _P]),
     "pico_swiglu_fwd": (c_int, [_P, _P, _P] + [_I64] * 5 + [c_int, _P]),
     "pico_swiglu_bwd": (c_int, [_P] * 5 + [_I64] * 7 + [c_int, _P]),
@@ -44,6 +44,7 @@ SIGNATURES = {
     "pico_cross_entropy_bwd": (c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, c_int, _P]),
     "pico_adamw": (c_int, [_P, _P, _P, c_int, _P, _P, _I64] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
     "pico_adamw_lp": (c_int, [_P, _P, c_int, _P, _P, _I64, c_int] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
+    "pico_adamw_multi": (c_int, [c_int, _P, _P, _P, _P, _P, _P, c_int, c_int] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
     "pico_convert_f32": (c_int, [_P, _P] + [_I64] * 7 + [c_int, _P]),
 }
 

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(kFwdThreads) void rmsnorm_fwd_kernel(
 template <typename T, int G, int NV>
 __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ rstd, T* __restrict__ dx, float* __restrict__ partial,
+    const float* __restrict__ rstd, const T* dres, T* dx, float* __restrict__ partial,
     int64_t rows, int hidden) {
   constexpr int V = io<T>::kVec;
   constexpr int GPB = kBwdThreads / G;
@@ -139,6 +139,12 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
         float o[V];
 #pragma unroll
         for (int e = 0; e < V; ++e) o[e] = r * (g[j][e] - xh[j][e] * c);
+        if (dres) {  // gradient that reached the residual stream directly; dx may alias it (same thread, same place)
+          float dr[V];
+          io<T>::load(dres + row * hidden + v * V, dr);
+#pragma unroll
+          for (int e = 0; e < V; ++e) o[e] += dr[e];
+        }
         io<T>::store(dx + row * hidden + v * V, o);
       }
     }
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
 template <typename T, int NV>
 __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
-    const float* __restrict__ rstd, T* __restrict__ dx, float* __restrict__ partial,
+    const float* __restrict__ rstd, const T* dres, T* dx, float* __restrict__ partial,
     int64_t rows, int hidden) {
   constexpr int V = io<T>::kVec;
   constexpr int NWAVE = kBwdWaveThreads / kWave;
@@ -185,7 +191,7 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
   const int nvec = hidden / V;
   const float inv_h = 1.f / static_cast<float>(hidden);
   float dw[NV][V], wv[NV][V];
-  u32x4 xr[NV], dr[NV];
+  u32x4 xr[NV], dr[NV], rr[NV];  // rr: the residual stream's own gradient, when there is one
   float rs;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
@@ -202,6 +208,7 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
       const int vc = v < nvec ? v : 0;
       xr[j] = *reinterpret_cast<const u32x4*>(x + r * hidden + vc * V);
       dr[j] = *reinterpret_cast<const u32x4*>(dy + r * hidden + vc * V);
+      if (dres) rr[j] = *reinterpret_cast<const u32x4*>(dres + r * hidden + vc * V);
     }
     rs = rstd[r];
   };
@@ -245,6 +252,12 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
         unpack(dr[j], dv);
 #pragma unroll
         for (int e = 0; e < V; ++e) o[e] = r * (dv[e] * wv[j][e] - xv[e] * r * c);
+        if (dres) {  // dx may alias dres: this lane read its part of the row before it writes it
+          float rv[V];
+          unpack(rr[j], rv);
+#pragma unroll
+          for (int e = 0; e < V; ++e) o[e] += rv[e];
+        }
         io<T>::store(dx + row * hidden + v * V, o);
       }
     }
@@ -281,8 +294,9 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
 
 // dweight[c] = sum_p partial[p][c]; 32 columns x 32 slices per block, every thread's loads issued together.
 constexpr int kReduceCols = 32;
+template <typename TW>
 __global__ __launch_bounds__(kReduceCols * 32) void rmsnorm_dw_reduce_kernel(
-    const float* __restrict__ partial, float* __restrict__ dweight, int nparts, int hidden) {
+    const float* __restrict__ partial, TW* __restrict__ dweight, int nparts, int hidden) {
   constexpr int kSlices = 32, kUnroll = 16;
   __shared__ float red[kSlices][kReduceCols + 1];
   const int c = threadIdx.x % kReduceCols;
@@ -307,8 +321,16 @@ __global__ __launch_bounds__(kReduceCols * 32) void rmsnorm_dw_reduce_kernel(
     float tot = 0.f;
 #pragma unroll
     for (int i = 0; i < kSlices; ++i) tot += red[i][c];
-    dweight[col] = tot;
+    dweight[col] = static_cast<TW>(tot);
   }
+}
+
+void launch_dw_reduce(const float* partial, void* dweight, int dweight_dtype, int nparts, int hidden, hipStream_t s) {
+  const dim3 grid(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)), block(kReduceCols * 32);
+  if (dweight_dtype == PICO_BF16)
+    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<__bf16>, grid, block, 0, s, partial, static_cast<__bf16*>(dweight), nparts, hidden);
+  else
+    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<float>, grid, block, 0, s, partial, static_cast<float*>(dweight), nparts, hidden);
 }
 
 int bwd_blocks(int64_t rows, int gpb) {
@@ -335,12 +357,12 @@ void launch_fwd(const void* x, const void* w, void* y, float* rstd, const void* 
 }
 
 template <typename T, int G, int NV>
-void launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, float* partial,
-                int blocks, int64_t rows, int hidden, hipStream_t s) {
+void launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx,
+                float* partial, int blocks, int64_t rows, int hidden, hipStream_t s) {
   const size_t lds = (kBwdThreads / G > 1) ? static_cast<size_t>(hidden) * sizeof(float) : 0;
   hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, G, NV>), dim3(blocks), dim3(kBwdThreads), lds, s,
                      static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), rstd,
-                     static_cast<T*>(dx), partial, rows, hidden);
+                     static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden);
 }
 
 template <typename T>
@@ -368,15 +390,15 @@ int dispatch_fwd(const void* x, const void* w, void* y, float* rstd, const void*
 }
 
 template <typename T>
-int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd, void* dx, float* partial,
-                 int64_t rows, int hidden, hipStream_t s, int* blocks_out) {
+int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx,
+                 float* partial, int64_t rows, int hidden, hipStream_t s, int* blocks_out) {
   const int nvec = hidden / io<T>::kVec;
   const int nv_wave = pick_nv((nvec + 63) / 64, 8);
 #define PICO_BWD(G, NV)                                                            \
   {                                                                                \
     const int blocks = bwd_blocks(rows, kBwdThreads / G);                          \
     *blocks_out = blocks;                                                          \
-    launch_bwd<T, G, NV>(dy, x, w, rstd, dx, partial, blocks, rows, hidden, s);    \
+    launch_bwd<T, G, NV>(dy, x, w, rstd, dres, dx, partial, blocks, rows, hidden, s); \
     return PICO_OK;                                                                \
   }
 #define PICO_BWD_WAVE(NV)                                                                              \
@@ -386,7 +408,7 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
     const size_t lds = static_cast<size_t>(kBwdWaveThreads / kWave - 1) * hidden * sizeof(float);      \
     hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV>), dim3(blocks), dim3(kBwdWaveThreads), lds, s,  \
                        static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w),  \
-                       rstd, static_cast<T*>(dx), partial, rows, hidden);                              \
+                       rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
     return PICO_OK;                                                                                    \
   }
   if (nv_wave && static_cast<size_t>(hidden) * 3 * sizeof(float) <= 65536) {
@@ -452,16 +474,16 @@ extern "C" int64_t pico_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t hidden
   return static_cast<int64_t>(kMaxBwdBlocks) * hidden * static_cast<int64_t>(sizeof(float));
 }
 
-extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd, void* dx,
-                                float* dweight, void* workspace, int64_t workspace_bytes, int64_t rows,
-                                int64_t hidden, int dtype, void* stream) {
+extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
+                                const void* dresidual, void* dx, void* dweight, int dweight_dtype, void* workspace,
+                                int64_t workspace_bytes, int64_t rows, int64_t hidden, int dtype, void* stream) {
   if (int rc = check_common("pico_rmsnorm_bwd", rows, hidden, dtype)) return rc;
+  if (dweight_dtype != PICO_BF16 && dweight_dtype != PICO_F32)
+    return fail(PICO_ERR_DTYPE, "pico_rmsnorm_bwd: dweight dtype code %d not supported", dweight_dtype);
   if (!dweight) return fail(PICO_ERR_NULL, "pico_rmsnorm_bwd: dweight is required");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (rows == 0) {  // empty sum: dweight = 0 (the reduce kernel with no partials writes zeros)
-    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)),
-                       dim3(kReduceCols * 32), 0, s, static_cast<const float*>(nullptr), dweight, 0,
-                       static_cast<int>(hidden));
+    launch_dw_reduce(nullptr, dweight, dweight_dtype, 0, static_cast<int>(hidden), s);
     return check_launch("pico_rmsnorm_bwd(empty)");
   }
   if (!dy || !x || !weight || !rstd || !dx || !workspace)
@@ -470,16 +492,16 @@ extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weigh
     return fail(PICO_ERR_WORKSPACE, "pico_rmsnorm_bwd: workspace has %lld bytes, needs %lld",
                 static_cast<long long>(workspace_bytes),
                 static_cast<long long>(pico_rmsnorm_bwd_workspace_bytes(rows, hidden)));
-  if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(workspace))
+  if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(workspace) ||
+      !aligned16(dresidual))
     return fail(PICO_ERR_ALIGN, "pico_rmsnorm_bwd: pointers must be 16-byte aligned");
   int blocks = 0;
   float* partial = static_cast<float*>(workspace);
   int rc = dtype == PICO_BF16
-               ? dispatch_bwd<__bf16>(dy, x, weight, rstd, dx, partial, rows, static_cast<int>(hidden), s, &blocks)
-               : dispatch_bwd<float>(dy, x, weight, rstd, dx, partial, rows, static_cast<int>(hidden), s, &blocks);
+               ? dispatch_bwd<__bf16>(dy, x, weight, rstd, dresidual, dx, partial, rows, static_cast<int>(hidden), s, &blocks)
+               : dispatch_bwd<float>(dy, x, weight, rstd, dresidual, dx, partial, rows, static_cast<int>(hidden), s, &blocks);
   if (rc) return rc;
   if (int lrc = check_launch("pico_rmsnorm_bwd")) return lrc;
-  hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)),
-                     dim3(kReduceCols * 32), 0, s, partial, dweight, blocks, static_cast<int>(hidden));
+  launch_dw_reduce(partial, dweight, dweight_dtype, blocks, static_cast<int>(hidden), s);
   return check_launch("pico_rmsnorm_bwd(dweight reduce)");
 }

@@ -32,14 +32,15 @@ __device__ __forceinline__ void store8(__bf16* p, const float (&in)[8]) { io<__b
 // p -= step_size * m / (sqrt(v) / sqrt(bc2) + eps),  step_size = lr / bc1.
 // TS is the type of the three states (the weight that is updated and both moments); param_lp, when given, receives
 // a bf16 copy of the updated weight.
+struct Hyper {
+  float decay, one_minus_b1, b2, one_minus_b2, step_size, inv_sqrt_bc2, eps, grad_scale;
+};
+
 template <typename TS, typename TG>
-__global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ param_lp, TS* __restrict__ master,
-                                                         const TG* __restrict__ grad, TS* __restrict__ exp_avg,
-                                                         TS* __restrict__ exp_avg_sq, int64_t n, float decay,
-                                                         float one_minus_b1, float b2, float one_minus_b2,
-                                                         float step_size, float inv_sqrt_bc2, float eps,
-                                                         float grad_scale) {
-  const int64_t i0 = (static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x) * kPerThread;
+__device__ __forceinline__ void adamw_block(__bf16* __restrict__ param_lp, TS* __restrict__ master,
+                                            const TG* __restrict__ grad, TS* __restrict__ exp_avg,
+                                            TS* __restrict__ exp_avg_sq, int64_t n, int64_t block, const Hyper& h) {
+  const int64_t i0 = (block * kThreads + threadIdx.x) * kPerThread;
   if (i0 >= n) return;
   float g[kPerThread], p[kPerThread], m[kPerThread], v[kPerThread];
   if (i0 + kPerThread <= n) {
@@ -58,12 +59,12 @@ __global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ pa
   }
 #pragma unroll
   for (int e = 0; e < kPerThread; ++e) {
-    const float ge = g[e] * grad_scale;
-    p[e] = p[e] * decay;
-    m[e] = m[e] + (ge - m[e]) * one_minus_b1;
-    v[e] = v[e] * b2 + ge * ge * one_minus_b2;
-    const float denom = __builtin_sqrtf(v[e]) * inv_sqrt_bc2 + eps;
-    p[e] = p[e] - step_size * (m[e] / denom);
+    const float ge = g[e] * h.grad_scale;
+    p[e] = p[e] * h.decay;
+    m[e] = m[e] + (ge - m[e]) * h.one_minus_b1;
+    v[e] = v[e] * h.b2 + ge * ge * h.one_minus_b2;
+    const float denom = __builtin_sqrtf(v[e]) * h.inv_sqrt_bc2 + h.eps;
+    p[e] = p[e] - h.step_size * (m[e] / denom);
   }
   if (i0 + kPerThread <= n) {
     store8(master + i0, p);
@@ -80,6 +81,40 @@ __global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ pa
   }
 }
 
+template <typename TS, typename TG>
+__global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ param_lp, TS* __restrict__ master,
+                                                         const TG* __restrict__ grad, TS* __restrict__ exp_avg,
+                                                         TS* __restrict__ exp_avg_sq, int64_t n, Hyper h) {
+  adamw_block<TS, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, blockIdx.x, h);
+}
+
+// Many tensors in one launch: the pointers travel in the kernel arguments (no table in device memory to keep alive),
+// and a workgroup finds its tensor by bisecting the running block count, which is uniform scalar work.
+constexpr int kMaxTensors = 48;
+struct TensorTable {
+  void* weight[kMaxTensors];
+  void* param_lp[kMaxTensors];
+  const void* grad[kMaxTensors];
+  void* exp_avg[kMaxTensors];
+  void* exp_avg_sq[kMaxTensors];
+  int64_t n[kMaxTensors];
+  unsigned block_start[kMaxTensors + 1];
+  int count;
+};
+
+template <typename TS, typename TG>
+__global__ __launch_bounds__(kThreads) void adamw_multi_kernel(TensorTable t, Hyper h) {
+  const unsigned bid = blockIdx.x;
+  int lo = 0, hi = t.count;   // block_start[lo] <= bid < block_start[hi]
+  while (hi - lo > 1) {
+    const int mid = (lo + hi) >> 1;
+    if (bid >= t.block_start[mid]) lo = mid; else hi = mid;
+  }
+  adamw_block<TS, TG>(static_cast<__bf16*>(t.param_lp[lo]), static_cast<TS*>(t.weight[lo]),
+                      static_cast<const TG*>(t.grad[lo]), static_cast<TS*>(t.exp_avg[lo]),
+                      static_cast<TS*>(t.exp_avg_sq[lo]), t.n[lo], bid - t.block_start[lo], h);
+}
+
 }  // namespace
 }  // namespace pico
 
@@ -87,40 +122,123 @@ using namespace pico;
 
 namespace {
 
+int hyper_check(const char* who, int grad_dtype, int64_t step) {
+  if (grad_dtype != PICO_BF16 && grad_dtype != PICO_F32)
+    return fail(PICO_ERR_DTYPE, "%s: gradient dtype code %d not supported", who, grad_dtype);
+  if (step < 1) return fail(PICO_ERR_SHAPE, "%s: step=%lld must be >= 1", who, static_cast<long long>(step));
+  return PICO_OK;
+}
+
+Hyper make_hyper(float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step, float grad_scale) {
+  // bias corrections in double, as torch computes them on the host
+  const double bc1 = 1.0 - __builtin_pow(static_cast<double>(beta1), static_cast<double>(step));
+  const double bc2 = 1.0 - __builtin_pow(static_cast<double>(beta2), static_cast<double>(step));
+  Hyper h;
+  h.decay = 1.f - lr * weight_decay;
+  h.one_minus_b1 = 1.f - beta1;
+  h.b2 = beta2;
+  h.one_minus_b2 = 1.f - beta2;
+  h.step_size = static_cast<float>(static_cast<double>(lr) / bc1);
+  h.inv_sqrt_bc2 = static_cast<float>(1.0 / __builtin_sqrt(bc2));
+  h.eps = eps;
+  h.grad_scale = grad_scale;
+  return h;
+}
+
+constexpr int64_t kPerBlock = static_cast<int64_t>(kThreads) * kPerThread;
+
 template <typename TS>
 int adamw_launch(const char* who, void* param_lp, TS* master, const void* grad, int grad_dtype, TS* exp_avg,
                  TS* exp_avg_sq, int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
                  int64_t step, float grad_scale, void* stream) {
-  if (grad_dtype != PICO_BF16 && grad_dtype != PICO_F32)
-    return fail(PICO_ERR_DTYPE, "%s: gradient dtype code %d not supported", who, grad_dtype);
-  if (n < 0 || step < 1) return fail(PICO_ERR_SHAPE, "%s: n=%lld must be >= 0 and step=%lld >= 1", who,
-                                     static_cast<long long>(n), static_cast<long long>(step));
+  if (int rc = hyper_check(who, grad_dtype, step)) return rc;
+  if (n < 0) return fail(PICO_ERR_SHAPE, "%s: n=%lld must be >= 0", who, static_cast<long long>(n));
   if (n == 0) return PICO_OK;
   if (!master || !grad || !exp_avg || !exp_avg_sq)
     return fail(PICO_ERR_NULL, "%s: the weight, grad, exp_avg and exp_avg_sq are required", who);
   if (!aligned16(param_lp) || !aligned16(master) || !aligned16(grad) || !aligned16(exp_avg) || !aligned16(exp_avg_sq))
     return fail(PICO_ERR_ALIGN, "%s: pointers must be 16-byte aligned", who);
-  // bias corrections in double, as torch computes them on the host
-  const double bc1 = 1.0 - __builtin_pow(static_cast<double>(beta1), static_cast<double>(step));
-  const double bc2 = 1.0 - __builtin_pow(static_cast<double>(beta2), static_cast<double>(step));
-  const float step_size = static_cast<float>(static_cast<double>(lr) / bc1);
-  const float inv_sqrt_bc2 = static_cast<float>(1.0 / __builtin_sqrt(bc2));
-  const float decay = 1.f - lr * weight_decay;
-  const int64_t per_block = static_cast<int64_t>(kThreads) * kPerThread;
-  const unsigned grid = static_cast<unsigned>((n + per_block - 1) / per_block);
+  const Hyper h = make_hyper(lr, beta1, beta2, eps, weight_decay, step, grad_scale);
+  const unsigned grid = static_cast<unsigned>((n + kPerBlock - 1) / kPerBlock);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (grad_dtype == PICO_BF16)
     hipLaunchKernelGGL((adamw_kernel<TS, __bf16>), dim3(grid), dim3(kThreads), 0, s, static_cast<__bf16*>(param_lp),
-                       master, static_cast<const __bf16*>(grad), exp_avg, exp_avg_sq, n, decay, 1.f - beta1, beta2,
-                       1.f - beta2, step_size, inv_sqrt_bc2, eps, grad_scale);
+                       master, static_cast<const __bf16*>(grad), exp_avg, exp_avg_sq, n, h);
   else
     hipLaunchKernelGGL((adamw_kernel<TS, float>), dim3(grid), dim3(kThreads), 0, s, static_cast<__bf16*>(param_lp),
-                       master, static_cast<const float*>(grad), exp_avg, exp_avg_sq, n, decay, 1.f - beta1, beta2,
-                       1.f - beta2, step_size, inv_sqrt_bc2, eps, grad_scale);
+                       master, static_cast<const float*>(grad), exp_avg, exp_avg_sq, n, h);
   return check_launch(who);
 }
 
+template <typename TS>
+int adamw_multi_launch(int count, void* const* weights, void* const* param_lps, const void* const* grads,
+                       void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int grad_dtype,
+                       const Hyper& h, hipStream_t s) {
+  const char* who = "pico_adamw_multi";
+  // validate everything before the first launch so that a rejected call has changed nothing
+  for (int i = 0; i < count; ++i) {
+    if (sizes[i] < 0) return fail(PICO_ERR_SHAPE, "%s: tensor %d has n=%lld", who, i, static_cast<long long>(sizes[i]));
+    if (sizes[i] == 0) continue;
+    if (!weights[i] || !grads[i] || !exp_avgs[i] || !exp_avg_sqs[i])
+      return fail(PICO_ERR_NULL, "%s: tensor %d: the weight, grad, exp_avg and exp_avg_sq are required", who, i);
+    if (!aligned16(weights[i]) || !aligned16(grads[i]) || !aligned16(exp_avgs[i]) || !aligned16(exp_avg_sqs[i]) ||
+        (param_lps && !aligned16(param_lps[i])))
+      return fail(PICO_ERR_ALIGN, "%s: tensor %d: pointers must be 16-byte aligned", who, i);
+    if ((sizes[i] + kPerBlock - 1) / kPerBlock > 0x7fffffff)
+      return fail(PICO_ERR_SHAPE, "%s: tensor %d is too large for one launch", who, i);
+  }
+  TensorTable t;
+  t.count = 0;
+  t.block_start[0] = 0;
+  auto flush = [&]() -> int {
+    if (t.count == 0) return PICO_OK;
+    const unsigned grid = t.block_start[t.count];
+    if (grad_dtype == PICO_BF16)
+      hipLaunchKernelGGL((adamw_multi_kernel<TS, __bf16>), dim3(grid), dim3(kThreads), 0, s, t, h);
+    else
+      hipLaunchKernelGGL((adamw_multi_kernel<TS, float>), dim3(grid), dim3(kThreads), 0, s, t, h);
+    t.count = 0;
+    return check_launch(who);
+  };
+  for (int i = 0; i < count; ++i) {
+    if (sizes[i] == 0) continue;
+    const uint64_t blocks = static_cast<uint64_t>((sizes[i] + kPerBlock - 1) / kPerBlock);
+    if (t.count == kMaxTensors || t.block_start[t.count] + blocks > 0x7fffffffu)
+      if (int rc = flush()) return rc;
+    const int j = t.count++;
+    t.weight[j] = weights[i];
+    t.param_lp[j] = param_lps ? param_lps[i] : nullptr;
+    t.grad[j] = grads[i];
+    t.exp_avg[j] = exp_avgs[i];
+    t.exp_avg_sq[j] = exp_avg_sqs[i];
+    t.n[j] = sizes[i];
+    t.block_start[j + 1] = t.block_start[j] + static_cast<unsigned>(blocks);
+  }
+  return flush();
+}
+
 }  // namespace
+
+extern "C" int pico_adamw_multi(int count, void* const* weights, void* const* param_lps, const void* const* grads,
+                                void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int state_dtype,
+                                int grad_dtype, float lr, float beta1, float beta2, float eps, float weight_decay,
+                                int64_t step, float grad_scale, void* stream) {
+  const char* who = "pico_adamw_multi";
+  if (int rc = hyper_check(who, grad_dtype, step)) return rc;
+  if (count < 0) return fail(PICO_ERR_SHAPE, "%s: count=%d must be >= 0", who, count);
+  if (count == 0) return PICO_OK;
+  if (!weights || !grads || !exp_avgs || !exp_avg_sqs || !sizes)
+    return fail(PICO_ERR_NULL, "%s: the pointer tables and sizes are required", who);
+  const Hyper h = make_hyper(lr, beta1, beta2, eps, weight_decay, step, grad_scale);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (state_dtype == PICO_F32)
+    return adamw_multi_launch<float>(count, weights, param_lps, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
+  if (state_dtype == PICO_BF16) {
+    if (param_lps) return fail(PICO_ERR_NULL, "%s: param_lps must be NULL when the state is bf16 (the weight is the parameter)", who);
+    return adamw_multi_launch<__bf16>(count, weights, nullptr, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
+  }
+  return fail(PICO_ERR_DTYPE, "%s: state dtype code %d not supported", who, state_dtype);
+}
 
 extern "C" int pico_adamw(void* param_lp, float* master, const void* grad, int grad_dtype, float* exp_avg,
                           float* exp_avg_sq, int64_t n, float lr, float beta1, float beta2, float eps,

@@ -18,8 +18,8 @@ class RMSNormFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy):
         x, weight, rstd = ctx.saved_tensors
-        dx, dw = ops.rmsnorm_bwd(dy, x, weight, rstd)
-        return dx, dw.to(weight.dtype), None, None
+        dx, dw = ops.rmsnorm_bwd(dy, x, weight, rstd, dw_dtype=weight.dtype)
+        return dx, dw, None, None
 
 
 class RMSNormResidualFunc(torch.autograd.Function):
@@ -34,10 +34,9 @@ class RMSNormResidualFunc(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dy, dh):
         h, weight, rstd = ctx.saved_tensors
-        dx, dw = ops.rmsnorm_bwd(dy, h, weight, rstd)
-        if dh is not None:
-            dx = dx + dh
-        return dx, dx, dw.to(weight.dtype), None
+        # dh, the gradient that reached h without passing the norm, is added inside the kernel
+        dx, dw = ops.rmsnorm_bwd(dy, h, weight, rstd, dresidual=dh, dw_dtype=weight.dtype)
+        return dx, dx, dw, None
 
 
 class RotaryFunc(torch.autograd.Function):
@@ -148,12 +147,12 @@ class QKVAttentionFunc(torch.autograd.Function):
     def forward(ctx, qkv, cos, sin, n_heads, n_kv_heads, head_dim, causal):
         B, S, _ = qkv.shape
         nq, nkv = n_heads * head_dim, n_kv_heads * head_dim
-        q = qkv[..., :nq].view(B, S, n_heads, head_dim).transpose(1, 2)
-        k = qkv[..., nq:nq + nkv].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
         v = qkv[..., nq + nkv:].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
-        # rotated copies in [B,S,H,D] memory (the projection output itself stays untouched: v is used as it lies)
-        q = ops.rope(q, cos, sin, 0, out=ops.empty_bshd(B, n_heads, S, head_dim, qkv.dtype, qkv.device))
-        k = ops.rope(k, cos, sin, 0, out=ops.empty_bshd(B, n_kv_heads, S, head_dim, qkv.dtype, qkv.device))
+        # q and k lie side by side, so one launch rotates both as Hq+Hkv heads into a [B,S,Hq+Hkv,D] copy (the
+        # projection output itself stays untouched: v is used as it lies)
+        qk = qkv[..., :nq + nkv].view(B, S, n_heads + n_kv_heads, head_dim).transpose(1, 2)
+        qk = ops.rope(qk, cos, sin, 0, out=ops.empty_bshd(B, n_heads + n_kv_heads, S, head_dim, qkv.dtype, qkv.device))
+        q, k = qk[:, :n_heads], qk[:, n_heads:]
         sm_scale = 1.0 / (head_dim ** 0.5)
         out, lse = ops.attn_fwd(q, k, v, sm_scale, causal, 0, out_dtype=qkv.dtype, bshd_out=True)
         ctx.save_for_backward(q, k, v, out, lse, cos, sin)
@@ -172,8 +171,8 @@ class QKVAttentionFunc(torch.autograd.Function):
         dv = dqkv[..., nq + nkv:].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
         do = dout.view(B, S, n_heads, head_dim).transpose(1, 2)
         ops.attn_bwd(do, q, k, v, lse, None, sm_scale, causal, 0, dq, dk, dv, out=out)
-        ops.rope(dq, cos, sin, 0, inverse=True, out=dq)
-        ops.rope(dk, cos, sin, 0, inverse=True, out=dk)
+        dqk = dqkv[..., :nq + nkv].view(B, S, n_heads + n_kv_heads, head_dim).transpose(1, 2)
+        ops.rope(dqk, cos, sin, 0, inverse=True, out=dqk)
         return dqkv, None, None, None, None, None, None
 
 

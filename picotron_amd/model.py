@@ -108,6 +108,11 @@ def _fused_projections() -> bool:
     return os.getenv("PICO_FUSED_PROJ", "1") != "0"
 
 
+def _fused_residual() -> bool:
+    """Residual adds inside the RMSNorm kernels on both passes (default); PICO_FUSED_RESIDUAL=0 keeps them apart."""
+    return os.getenv("PICO_FUSED_RESIDUAL", "1") != "0"
+
+
 def _fused_weight(owner, name, linears):
     """The [sum(out_i), in] buffer that the weights of `linears` alias, row block by row block.  Built on first use
     and rebuilt whenever the Parameters were moved or cast since (``model.to(...)`` gives them fresh storage); the
@@ -251,6 +256,18 @@ class DecoderLayer(nn.Module):
         x = x + self.mlp(self.post_attention_layernorm(x))
         return x
 
+    def forward_chained(self, branch, residual, attention_mask=None, position_ids=None):
+        """The same layer with the residual stream carried beside the branch output, the way flash-attn's
+        layer_norm_fn(residual=..., prenorm=True) is meant to be chained: the layer's input is `branch + residual`
+        (`residual` None: just `branch`), each add happens inside the norm kernel that follows it, and the layer
+        returns (mlp output, residual stream before it) for the next norm to add.  Forward values are those of
+        forward(); in the backward the gradient of the residual stream enters the norm's backward kernel, so no
+        separate add runs on either pass."""
+        y, residual = self.input_layernorm(branch, residual=residual, prenorm=True)
+        a = self.attention(y, self.cos, self.sin, attention_mask, position_ids)
+        y, residual = self.post_attention_layernorm(a, residual=residual, prenorm=True)
+        return self.mlp(y), residual
+
 
 class Embedding(nn.Module):
     def __init__(self, num_embeddings, embedding_dim, padding_idx=None):
@@ -314,7 +331,14 @@ class Llama(nn.Module):
 
     def forward(self, input_ids, attention_mask=None, position_ids: torch.Tensor = None):
         x = self.embedding(input_ids)
-        for layer in self.decoder_layers:
-            x = layer(x)
-        x = self.final_norm(x)
+        if _fused_residual() and isinstance(self.final_norm, TritonRMSNorm) and all(
+                isinstance(l.input_layernorm, TritonRMSNorm) for l in self.decoder_layers):
+            residual = None
+            for layer in self.decoder_layers:
+                x, residual = layer.forward_chained(x, residual)
+            x = self.final_norm(x, residual=residual)
+        else:
+            for layer in self.decoder_layers:
+                x = layer(x)
+            x = self.final_norm(x)
         return self.final_proj(x)

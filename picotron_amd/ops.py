@@ -56,21 +56,30 @@ def rmsnorm_fwd(x: torch.Tensor, weight: torch.Tensor, eps: float, cast_then_sca
     return y, rstd, res_out
 
 
-def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor):
-    """Returns (dx in x.dtype, dweight fp32 [hidden])."""
-    _dev(dy, x, weight, rstd)
+def rmsnorm_bwd(dy: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, rstd: torch.Tensor,
+                dresidual: Optional[torch.Tensor] = None, dw_dtype=torch.float32):
+    """Returns (dx in x.dtype, dweight [hidden] in dw_dtype).  `dresidual` (x's shape and dtype), when given, is added
+    to dx inside the kernel: the gradient that reached the residual stream directly."""
+    _dev(dy, x, weight, rstd, dresidual)
     hidden = x.size(-1)
     xc, dyc = x.contiguous(), dy.contiguous()
     if dyc.dtype != xc.dtype:
         dyc = dyc.to(xc.dtype)
+    if dresidual is not None:
+        if dresidual.shape != x.shape:
+            raise RuntimeError("rmsnorm_bwd: dresidual must have x's shape")
+        dresidual = dresidual.contiguous()
+        if dresidual.dtype != xc.dtype:
+            dresidual = dresidual.to(xc.dtype)
     w = weight.to(x.dtype).contiguous() if weight.dtype != x.dtype else weight.contiguous()
     rows = xc.numel() // hidden if hidden else 0
     dx = torch.empty_like(xc)
-    dw = torch.empty(hidden, dtype=torch.float32, device=x.device)
+    dw = torch.empty(hidden, dtype=dw_dtype, device=x.device)
     ws_bytes = _lib.lib().pico_rmsnorm_bwd_workspace_bytes(rows, hidden)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=x.device)
-    check(_lib.lib().pico_rmsnorm_bwd(_ptr(dyc), _ptr(xc), _ptr(w), _ptr(rstd), _ptr(dx), _ptr(dw), _ptr(ws), ws_bytes,
-                                      rows, hidden, _dt(x, "rmsnorm_bwd"), _stream()))
+    check(_lib.lib().pico_rmsnorm_bwd(_ptr(dyc), _ptr(xc), _ptr(w), _ptr(rstd), _ptr(dresidual), _ptr(dx), _ptr(dw),
+                                      _dt(dw, "rmsnorm_bwd dweight"), _ptr(ws), ws_bytes, rows, hidden,
+                                      _dt(x, "rmsnorm_bwd"), _stream()))
     return dx, dw
 
 
@@ -403,6 +412,69 @@ def adamw_lp_(param: torch.Tensor, grad: torch.Tensor, exp_avg: torch.Tensor, ex
     check(_lib.lib().pico_adamw_lp(_ptr(param), _ptr(grad), _dt(grad, "grad"), _ptr(exp_avg), _ptr(exp_avg_sq), n,
                                    _dt(param, "param"), float(lr), float(beta1), float(beta2), float(eps),
                                    float(weight_decay), int(step), float(grad_scale), _stream()))
+
+
+class AdamWMultiPlan:
+    """The AdamW step for a fixed list of tensors in as few launches as they fit (48 tensors each).  Weights, moments
+    and sizes are checked and their pointer tables built once; a step only fills in the gradients' addresses, so its
+    host cost is a fraction of a millisecond for a few hundred tensors.  All weights and moments share one dtype:
+    fp32 (master weights; `param_lps` optionally lists the bf16 parameters to rewrite, None entries allowed) or bf16
+    (the weights are the parameters; `param_lps` must be None).  The plan keeps the tensors alive."""
+
+    def __init__(self, weights, exp_avgs, exp_avg_sqs, param_lps=None):
+        count = len(weights)
+        if count == 0 or not (len(exp_avgs) == len(exp_avg_sqs) == count) or (param_lps is not None and len(param_lps) != count):
+            raise RuntimeError("adamw_multi_: the lists must have one entry per tensor (and at least one)")
+        sdt = weights[0].dtype
+        for i in range(count):
+            w, m, v = weights[i], exp_avgs[i], exp_avg_sqs[i]
+            _dev(w, m, v)
+            n = w.numel()
+            for t, what in ((w, "weight"), (m, "exp_avg"), (v, "exp_avg_sq")):
+                if t.dtype != sdt or not t.is_contiguous() or t.numel() != n:
+                    raise RuntimeError(f"adamw_multi_: tensor {i}: {what} must be a contiguous {sdt} tensor of {n} elements")
+            if param_lps is not None and param_lps[i] is not None:
+                lp = param_lps[i]
+                _dev(lp)
+                if lp.dtype != torch.bfloat16 or not lp.is_contiguous() or lp.numel() != n:
+                    raise RuntimeError(f"adamw_multi_: tensor {i}: param_lp must be a contiguous bf16 tensor of {n} elements")
+        self.count = count
+        self._keep = (list(weights), list(exp_avgs), list(exp_avg_sqs), list(param_lps) if param_lps is not None else None)
+        self._arr = ctypes.c_void_p * count
+        table = lambda ts: self._arr(*[t.data_ptr() if t is not None else None for t in ts])
+        self._w, self._m, self._v = table(weights), table(exp_avgs), table(exp_avg_sqs)
+        self._lp = table(param_lps) if param_lps is not None else None
+        self._numel = [w.numel() for w in weights]
+        self._sizes = (ctypes.c_int64 * count)(*self._numel)
+        self._state_dt = _dt(weights[0], "weight")
+
+    def step(self, grads, step: int, lr: float, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8,
+             weight_decay: float = 0.01, grad_scale: float = 1.0) -> None:
+        if len(grads) != self.count:
+            raise RuntimeError("adamw_multi_: the lists must have one entry per tensor")
+        gdt = grads[0].dtype
+        keep = []   # contiguous copies of gradients must outlive the launch call
+        g_arr = self._arr()
+        for i, g in enumerate(grads):
+            if not g.is_cuda:
+                _dev(g)
+            if g.dtype != gdt or g.numel() != self._numel[i]:
+                raise RuntimeError(f"adamw_multi_: tensor {i}: grad must have dtype {gdt} and {self._numel[i]} elements")
+            if not g.is_contiguous():
+                g = g.contiguous()
+                keep.append(g)
+            g_arr[i] = g.data_ptr()
+        check(_lib.lib().pico_adamw_multi(self.count, self._w, self._lp, g_arr, self._m, self._v, self._sizes,
+                                          self._state_dt, _dt(grads[0], "grad"), float(lr), float(beta1), float(beta2),
+                                          float(eps), float(weight_decay), int(step), float(grad_scale), _stream()))
+
+
+def adamw_multi_(weights, grads, exp_avgs, exp_avg_sqs, step: int, lr: float, beta1: float = 0.9, beta2: float = 0.999,
+                 eps: float = 1e-8, weight_decay: float = 0.01, grad_scale: float = 1.0, param_lps=None) -> None:
+    """One AdamW step for a list of tensors (see AdamWMultiPlan, which a training loop should build once)."""
+    if len(weights) == 0 and len(grads) == 0:
+        return
+    AdamWMultiPlan(weights, exp_avgs, exp_avg_sqs, param_lps).step(grads, step, lr, beta1, beta2, eps, weight_decay, grad_scale)
 
 
 def _ce_check(logits: torch.Tensor, targets: torch.Tensor):

@@ -28,6 +28,7 @@ class FusedAdamW:
                 raise RuntimeError("FusedAdamW: parameters must be contiguous bf16 / fp32 tensors on the GPU")
         self.lr, self.betas, self.eps, self.weight_decay = lr, betas, eps, weight_decay
         self.step_count = 0
+        self._plans = {}
         dev = self.params[0].device
         # every tensor starts on a multiple of 8 elements so that all kernel accesses are 16-byte aligned
         self.offsets, total = [], 0
@@ -103,7 +104,36 @@ class FusedAdamW:
             self._open = False
             return
         self.step_count += 1
-        for p, off in zip(self.params, self.offsets):
-            if p.grad is None:
-                continue
-            self._update(p, off, p.grad, grad_scale)
+        live = tuple(i for i, p in enumerate(self.params) if p.grad is not None)
+        if not live:
+            return
+        hyper = (self.step_count, self.lr, self.betas[0], self.betas[1], self.eps, self.weight_decay, grad_scale)
+        # one launch table per gradient dtype; the tables (everything but the gradients' addresses) are built once per
+        # set of live parameters and reused, so the host side of a step stays far below the kernel's own time
+        by_dtype = {}
+        for i in live:
+            by_dtype.setdefault(self.params[i].grad.dtype, []).append(i)
+        for gdt, idx in by_dtype.items():
+            key = (gdt, tuple(idx))
+            plan = self._plans.get(key)
+            if plan is None or any(self.params[i].data_ptr() != ptr for i, ptr in zip(idx, plan.param_ptrs)):
+                plan = self._plans[key] = self._make_plan(idx)
+            plan.step([self.params[i].grad for i in idx], *hyper)
+            if self.master_weights:
+                for i in idx:
+                    p = self.params[i]
+                    if p.dtype == torch.float32:
+                        off = self.offsets[i]
+                        p.copy_(self.master[off:off + p.numel()].view_as(p))
+
+    def _make_plan(self, idx):
+        ps = [self.params[i] for i in idx]
+        ms = [self.exp_avg[self.offsets[i]:self.offsets[i] + self.params[i].numel()] for i in idx]
+        vs = [self.exp_avg_sq[self.offsets[i]:self.offsets[i] + self.params[i].numel()] for i in idx]
+        if self.master_weights:
+            ws = [self.master[self.offsets[i]:self.offsets[i] + self.params[i].numel()] for i in idx]
+            plan = ops.AdamWMultiPlan(ws, ms, vs, [p.detach().view(-1) if p.dtype == torch.bfloat16 else None for p in ps])
+        else:
+            plan = ops.AdamWMultiPlan([p.detach().view(-1) for p in ps], ms, vs)
+        plan.param_ptrs = [p.data_ptr() for p in ps]   # a parameter that was moved or cast since invalidates the plan
+        return plan

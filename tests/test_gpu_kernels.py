@@ -82,6 +82,26 @@ def test_rmsnorm_bwd(ops, device, rows, hidden, dtype):
     assert rel_l2(dw, want_dw) <= 1e-5
 
 
+@pytest.mark.parametrize("rows,hidden", [(7, 576), (300, 2048), (33, 8192), (1030, 1024)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_rmsnorm_bwd_adds_residual_gradient_and_rounds_dweight(ops, device, rows, hidden, dtype):
+    """dresidual is added to dx inside the kernel (fp32 sum, one rounding) and dweight comes back in the requested
+    dtype: against the oracle's dx + dresidual, and bit-identical in dweight (after rounding) to the call without."""
+    x, dy, dr = (rnd(rows, hidden, seed=s_, dtype=dtype) for s_ in (6, 7, 12))
+    w = (1 + 0.1 * rnd(hidden, seed=8)).to(dtype)
+    rstd = torch.rsqrt(x.float().pow(2).mean(-1) + 1e-5)
+    dev = lambda t: t.to(device)
+    dx0, dw0 = ops.rmsnorm_bwd(dev(dy), dev(x), dev(w), dev(rstd))
+    dx, dw = ops.rmsnorm_bwd(dev(dy), dev(x), dev(w), dev(rstd), dresidual=dev(dr), dw_dtype=dtype)
+    want_dx, _ = OL.rmsnorm_backward(dy, x, w, 1e-5)
+    assert rel_l2(dx, want_dx.float() + dr.float()) <= (1e-5 if dtype == torch.float32 else 4e-3)
+    assert dw.dtype == dtype and torch.equal(dw.cpu(), dw0.cpu().to(dtype))
+    # the sum is taken before rounding: never further from the exact sum than rounding it once
+    exact = dx0.double().cpu() * 0 + (want_dx.double() + dr.double())
+    if dtype == torch.bfloat16:
+        assert ((dx.double().cpu() - exact).abs() <= exact.abs() * 2.0 ** -8 + want_dx.double().abs() * 2.0 ** -7 + 1e-6).all()
+
+
 # ------------------------------------------------------------------------------------ RoPE
 @pytest.mark.parametrize("B,H,S,D", [(2, 3, 17, 64), (1, 4, 33, 128), (1, 2, 5, 16)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
@@ -469,6 +489,37 @@ def test_adamw_lp_kernel_against_oracle(ops, device, n, grad_dtype):
             diff = (got.cpu().float() - w.float()).abs()
             assert (diff <= w.float().abs() * 2.0 ** -7 + w.float().abs().mean() * 2.0 ** -14).all()
             assert (diff != 0).sum().item() <= max(1, 0.03 * n)
+
+
+@pytest.mark.parametrize("state_dtype", [torch.bfloat16, torch.float32])
+def test_adamw_multi_equals_one_call_per_tensor(ops, device, state_dtype):
+    """pico_adamw_multi over 61 tensors (more than one launch's table holds; sizes 0, 1, odd and many blocks) leaves
+    every state bit-identical to pico_adamw / pico_adamw_lp called once per tensor."""
+    g = torch.Generator().manual_seed(17)
+    sizes = [0, 1, 5, 2048, 2049, 40000] + [int(x) for x in torch.randint(1, 30000, (55,), generator=g)]
+    lp = state_dtype == torch.bfloat16
+    def fresh():
+        gg = torch.Generator().manual_seed(18)
+        mk = lambda n, pos=False: (torch.rand(n, generator=gg) if pos else torch.randn(n, generator=gg)).to(state_dtype).to(device)
+        return ([mk(n) for n in sizes], [mk(n) for n in sizes], [mk(n, True) for n in sizes],
+                [torch.randn(n, generator=gg).bfloat16().to(device) for n in sizes])
+    w1, m1, v1, gr = fresh()
+    w2, m2, v2, _ = fresh()
+    lp1 = None if lp else [torch.empty(n, dtype=torch.bfloat16, device=device) if i % 3 else None for i, n in enumerate(sizes)]
+    lp2 = None if lp else [torch.empty(n, dtype=torch.bfloat16, device=device) if i % 3 else None for i, n in enumerate(sizes)]
+    hyper = (3, 2e-3, 0.9, 0.95, 1e-8, 0.1, 0.5)
+    ops.adamw_multi_(w1, gr, m1, v1, *hyper, param_lps=lp1)
+    for i in range(len(sizes)):
+        if lp:
+            ops.adamw_lp_(w2[i], gr[i], m2[i], v2[i], *hyper)
+        else:
+            ops.adamw_(lp2[i], w2[i], gr[i], m2[i], v2[i], *hyper)
+    for i in range(len(sizes)):
+        assert torch.equal(w1[i], w2[i]) and torch.equal(m1[i], m2[i]) and torch.equal(v1[i], v2[i]), sizes[i]
+        if not lp and lp1[i] is not None:
+            assert torch.equal(lp1[i], lp2[i])
+    with pytest.raises(RuntimeError, match="one entry per tensor"):
+        ops.adamw_multi_(w1, gr[:-1], m1, v1, *hyper)
 
 
 def test_fused_adamw_without_master_weights_follows_torch_fused_adamw(device):

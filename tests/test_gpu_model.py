@@ -249,3 +249,31 @@ def test_fused_projections_match_separate_projections(pgm1, device):
     assert abs(grads["0"][0] - grads["1"][0]) <= 2e-3
     for n, g0 in grads["0"][1].items():
         assert rel_l2(grads["1"][1][n], g0) <= 2e-2, n
+
+
+def test_chained_residual_stream_matches_separate_adds(pgm1, device):
+    """PICO_FUSED_RESIDUAL: residual adds inside the RMSNorm kernels (forward: layer_norm_fn's residual= / prenorm=
+    chaining; backward: the residual stream's gradient enters the norm's backward kernel) must give the loss and
+    parameter gradients of the layer written as x + f(norm(x)) with torch adds."""
+    from picotron_amd.functional import cross_entropy
+    from picotron_amd.model import Llama
+    cfg = OM.LlamaShape(256, 4, 2, 512, 1024, 3, 128)
+    ids, tgt = OM.synthetic_batch(cfg.vocab_size, 2, 128, seed=5)
+    ids, tgt = ids.to(device), tgt.to(device)
+    res = {}
+    try:
+        for mode in ("0", "1"):
+            os.environ["PICO_FUSED_RESIDUAL"] = mode
+            torch.manual_seed(0)
+            m = Llama(cfg).to(device).to(torch.bfloat16)
+            logits = m(ids)
+            loss = cross_entropy(logits.view(-1, cfg.vocab_size), tgt.reshape(-1))
+            loss.backward()
+            res[mode] = (loss.item(), logits.detach().float().cpu(), {n: p.grad.float().cpu() for n, p in m.named_parameters()})
+    finally:
+        os.environ.pop("PICO_FUSED_RESIDUAL", None)
+    assert abs(res["0"][0] - res["1"][0]) <= 2e-3
+    assert rel_l2(res["1"][1], res["0"][1]) <= 1e-2
+    for n, g0 in res["0"][2].items():
+        assert res["1"][2][n].dtype == g0.dtype
+        assert rel_l2(res["1"][2][n], g0) <= 2e-2, n
