@@ -20,12 +20,16 @@ struct FwdParams {
   int pair_order;  // dispatch order of the query tiles, see the kernel
 };
 
+#ifndef PICO_FWD_KDEPTH
+#define PICO_FWD_KDEPTH (D >= 128 ? 2 : 0)
+#endif
 template <int D, int QB, int NW, int KT>
 struct FwdCfg {
   static constexpr int kThreads = 64 * NW;
   static constexpr int BM = 32 * QB * NW;  // queries per workgroup
   static constexpr int BN = 64;            // keys per compute step
   static constexpr int kKT = KT;           // keys per staged LDS tile (a multiple of BN), double-buffered
+  static constexpr int kKDepth = PICO_FWD_KDEPTH;  // K fragments in flight from LDS ahead of the MFMA that uses them (0: compiler's order)
   static constexpr int LDK = D + 8;        // K tile pitch: 16-byte row reads hit distinct banks
 #ifndef PICO_FWD_LDVPAD
 #define PICO_FWD_LDVPAD 8
@@ -42,6 +46,15 @@ struct FwdCfg {
 
 #ifndef PICO_FWD_KT8
 #define PICO_FWD_KT8 64
+#endif
+#ifndef PICO_FWD_KT128
+#define PICO_FWD_KT128 128
+#endif
+#ifndef PICO_FWD_CFG128
+#define PICO_FWD_CFG128 128, 1, 8, PICO_FWD_KT128
+#endif
+#ifndef PICO_FWD_CFG64
+#define PICO_FWD_CFG64 64, 1, 8, PICO_FWD_KT8
 #endif
 #ifndef PICO_FWD_ATTR
 #define PICO_FWD_ATTR
@@ -200,14 +213,41 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
         if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
         // ---- S^T[key][query] for 64 keys x 32 queries
         f32x16 s_acc[BN / 32];
+        // D = 128: the K fragments are fetched from LDS a fixed number of MFMAs ahead of their use.  An LDS read
+        // takes several MFMA times to come back, so a read issued right before its MFMA leaves the matrix pipe
+        // waiting for it (measured: +5 %).  At D = 64 the softmax arithmetic, not this wait, paces the loop, and the
+        // compiler's own order is 2 % faster.
+        if constexpr (C::kKDepth > 0) {
+          constexpr int kSteps = (BN / 32) * (D / 16), kDepth = C::kKDepth < kSteps ? C::kKDepth : kSteps;
+          bf16x8 kf[kSteps];
 #pragma unroll
-        for (int mb = 0; mb < BN / 32; ++mb) {
+          for (int j = 0; j < kSteps; ++j)
+            kf[j] = *reinterpret_cast<const bf16x8*>(&sKs[(32 * (j / (D / 16)) + n) * LDK + 16 * (j % (D / 16)) + 8 * h]);
 #pragma unroll
-          for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+          for (int mb = 0; mb < BN / 32; ++mb) {
 #pragma unroll
-          for (int s = 0; s < D / 16; ++s) {
-            const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
-            s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
+            for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+#pragma unroll
+            for (int s = 0; s < D / 16; ++s) s_acc[mb] = mfma32(kf[mb * (D / 16) + s], qf[qb][s], s_acc[mb]);
+          }
+          // scheduling groups: kDepth LDS reads, then one MFMA and one read in turn, then the last kDepth MFMAs
+          __builtin_amdgcn_sched_group_barrier(0x100, kDepth, 0);
+#pragma unroll
+          for (int j = 0; j < kSteps - kDepth; ++j) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, kDepth, 0);
+        } else {
+#pragma unroll
+          for (int mb = 0; mb < BN / 32; ++mb) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s_acc[mb][i] = 0.f;
+#pragma unroll
+            for (int s = 0; s < D / 16; ++s) {
+              const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
+              s_acc[mb] = mfma32(kf, qf[qb][s], s_acc[mb]);
+            }
           }
         }
         // ---- mask (only for tiles that straddle the diagonal or the end of K)
@@ -384,12 +424,12 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
   if (desc->D == 64) {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
-    if (groups(256) >= 512) rc = launch<64, 1, 8, PICO_FWD_KT8>(p, s);
+    if (groups(256) >= 512) rc = launch<PICO_FWD_CFG64>(p, s);
     else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
     else rc = launch<64, 1, 2, 64>(p, s);
   } else {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
-    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<128, 1, 8, 64>(p, s);
+    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<PICO_FWD_CFG128>(p, s);
     else rc = launch<128, 1, 4, 64>(p, s);
   }
   if (rc) return rc;
