@@ -263,22 +263,26 @@ def bandwidth_extras(torch, ops, iters=50):
     lse_c = ops.cross_entropy_fwd(torch.randn(T, Vc, device=dev).to(bf), tg)[1]
     run("cross_entropy_bwd", lambda: (torch.randn(T, Vc, device=dev).to(bf),),
         lambda lg: ops.cross_entropy_bwd(lg, tg, lse_c, one), 2 * T * Vc * 2, 2)
-    # AdamW on 64 Mi bf16 parameters: 28 bytes per parameter with fp32 master weights and moments, 14 with bf16 state
+    # AdamW on 64 Mi bf16 parameters: 28 bytes per parameter with fp32 master weights and moments, 22 with fp32 moments
+    # only, 14 with bf16 state
     n = 64 * 1024 * 1024
     run("adamw", lambda: (torch.zeros(n, device=dev, dtype=bf), torch.randn(n, device=dev), torch.randn(n, device=dev).to(bf),
                           torch.zeros(n, device=dev), torch.zeros(n, device=dev)),
         lambda p_, m_, g_, ea, eas: ops.adamw_(p_, m_, g_, ea, eas, 1, 1e-3), 28 * n, 1)
-    run("adamw_lp", lambda: tuple(torch.randn(n, device=dev).to(bf) for _ in range(3)) + (torch.rand(n, device=dev).to(bf),),
+    run("adamw_lp_fp32_moments", lambda: (torch.randn(n, device=dev).to(bf), torch.randn(n, device=dev).to(bf), torch.randn(n, device=dev), torch.rand(n, device=dev)),
+        lambda p_, g_, ea, eas: ops.adamw_lp_(p_, g_, ea, eas, 1, 1e-3), 22 * n, 1)
+    run("adamw_lp_bf16_moments", lambda: tuple(torch.randn(n, device=dev).to(bf) for _ in range(3)) + (torch.rand(n, device=dev).to(bf),),
         lambda p_, g_, ea, eas: ops.adamw_lp_(p_, g_, ea, eas, 1, 1e-3), 14 * n, 1)
     return res
 
 
-def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, master_weights=False):
+def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, adamw="fp32_moments"):
     """configs[2]: SmolLM-1.7B-shaped training step (24 layers, h 2048, 32 heads of 64, I 8192, V 49152), mbs 4, seq 1024;
     configs[3]: Llama-2-7B-shaped step (32 layers, h 4096, 32 heads of 128, I 11008, V 32000), mbs 1, seq 4096.
-    bf16 parameters, random init, synthetic tokens.  AdamW state as the reference holds it (train.py:209: AdamW on the
-    bf16 parameters, so bf16 moments and an in-place bf16 update) or, with master_weights, fp32 master weights and
-    moments."""
+    bf16 parameters, random init, synthetic tokens.  adamw selects the optimizer's memory layout:
+    "fp32_moments" (the named configuration: bf16 parameters updated in place, fp32 AdamW state), "fp32_master" (an
+    fp32 master copy of every parameter as well) or "reference" (the state as the reference holds it, train.py:209:
+    AdamW on the bf16 parameters, so bf16 moments)."""
     import torch.nn.functional as F
 
     import picotron_amd.process_group_manager as pgm
@@ -297,8 +301,11 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, master_weigh
     # one fused pass per parameter tensor (picotron_amd.optim.FusedAdamW over pico_adamw_lp / pico_adamw)
     from picotron_amd.functional import cross_entropy
     from picotron_amd.optim import FusedAdamW
-    opt = FusedAdamW(model.parameters(), lr=3e-4, master_weights=master_weights,
-                     overlap_with_backward=os.getenv("PICO_BENCH_OVERLAP", "0") == "1")
+    layouts = {"fp32_moments": (dict(master_weights=False, state_dtype=torch.float32), "bf16 parameters updated in place, fp32 moments"),
+               "fp32_master": (dict(master_weights=True), "fp32 master weights and moments"),
+               "reference": (dict(master_weights=False), "bf16 moments, bf16 parameter updated in place (the reference's layout)")}
+    opt = FusedAdamW(model.parameters(), lr=3e-4, overlap_with_backward=os.getenv("PICO_BENCH_OVERLAP", "0") == "1",
+                     **layouts[adamw][0])
     ids, tgt = synthetic_batch(cfg.vocab_size, mbs, seq, seed=0)
     ids, tgt = ids.cuda(), tgt.cuda()
 
@@ -323,7 +330,7 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, master_weigh
     fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, seq)
     res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
            "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
-           "adamw_state": "fp32 master weights and moments" if master_weights else "bf16 moments, bf16 parameter updated in place (the reference's layout)",
+           "adamw_state": layouts[adamw][1],
            "note": "attention / RMSNorm / RoPE / SwiGLU / cross-entropy / AdamW on the HIP kernels; embedding, projections "
                    "and residual adds on torch"}
     del model, opt
@@ -508,7 +515,8 @@ def main():
         extras["configs4_long_context_rank7_of_8"] = long_context_extra(torch, ops)
         if not args.no_train:
             extras["smollm_1p7b_train_step"] = train_step_extra(torch, "smollm_1p7b")
-            extras["smollm_1p7b_train_step_fp32_master"] = train_step_extra(torch, "smollm_1p7b", master_weights=True)
+            extras["smollm_1p7b_train_step_fp32_master"] = train_step_extra(torch, "smollm_1p7b", adamw="fp32_master")
+            extras["smollm_1p7b_train_step_reference_adamw_layout"] = train_step_extra(torch, "smollm_1p7b", adamw="reference")
             extras["llama2_7b_train_step"] = train_step_extra(torch, "llama2_7b", steps=4, warmup=2)
 
     line = {

@@ -222,26 +222,28 @@ int pico_cross_entropy_bwd(const void* logits, const int64_t* targets, const flo
 int pico_adamw(void* param_lp, float* master, const void* grad, int grad_dtype, float* exp_avg, float* exp_avg_sq,
                int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step,
                float grad_scale, void* stream);
-/* The same step with the state held as the reference holds it for a bf16 model (train.py:209 builds AdamW on the
- * bf16 parameters, so torch keeps exp_avg and exp_avg_sq in bf16 and updates the bf16 parameter itself): param,
- * exp_avg, exp_avg_sq are [n] of `dtype` (PICO_BF16), updated in place; the arithmetic is fp32 and each state is
- * rounded once per step (what torch's fused AdamW does; its default for-each path rounds after every operation).
+/* The same step on the bf16 parameter itself, no master copy: param [n] of param_dtype (PICO_BF16) is read, updated
+ * and rounded once in place.  exp_avg / exp_avg_sq are [n] of state_dtype:
+ *   PICO_F32   fp32 moments ("bf16 parameters with fp32 AdamW state"), 22 bytes of traffic per parameter;
+ *   PICO_BF16  the state as the reference holds it (train.py:209 builds AdamW on the bf16 parameters, so torch keeps
+ *              exp_avg and exp_avg_sq in bf16), 14 bytes; fp32 arithmetic and one rounding per state, which is what
+ *              torch's fused AdamW does (its default for-each path rounds after every operation).
  */
-int pico_adamw_lp(void* param, const void* grad, int grad_dtype, void* exp_avg, void* exp_avg_sq, int64_t n, int dtype,
-                  float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step, float grad_scale,
-                  void* stream);
+int pico_adamw_lp(void* param, const void* grad, int grad_dtype, void* exp_avg, void* exp_avg_sq, int64_t n,
+                  int param_dtype, int state_dtype, float lr, float beta1, float beta2, float eps, float weight_decay,
+                  int64_t step, float grad_scale, void* stream);
 /* The step for `count` tensors at once (what torch's for-each / fused AdamW does for the whole parameter list of
  * train.py:209): host arrays of `count` device pointers and sizes; the library packs them into the arguments of as
  * few launches as they fit (48 tensors each), so a model's ~200 parameter tensors cost 5 launches instead of 200.
- * state_dtype PICO_F32: weights are the fp32 master weights and param_lps (the array or single entries may be NULL)
- * receive their bf16 copies, as pico_adamw; PICO_BF16: weights are the bf16 parameters themselves and param_lps must
- * be NULL, as pico_adamw_lp.  All gradients share grad_dtype.  Tensors of size 0 are skipped.  Every tensor is
- * checked before the first launch: a rejected call has changed nothing.
+ * (weight_dtype, state_dtype) = (PICO_F32, PICO_F32): weights are the fp32 master weights and param_lps (the array
+ * or single entries may be NULL) receive their bf16 copies, as pico_adamw; (PICO_BF16, PICO_F32 or PICO_BF16): weights
+ * are the bf16 parameters themselves and param_lps must be NULL, as pico_adamw_lp.  All gradients share grad_dtype.
+ * Tensors of size 0 are skipped.  Every tensor is checked before the first launch: a rejected call has changed nothing.
  */
 int pico_adamw_multi(int count, void* const* weights, void* const* param_lps, const void* const* grads,
-                     void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int state_dtype,
-                     int grad_dtype, float lr, float beta1, float beta2, float eps, float weight_decay, int64_t step,
-                     float grad_scale, void* stream);
+                     void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int weight_dtype,
+                     int state_dtype, int grad_dtype, float lr, float beta1, float beta2, float eps, float weight_decay,
+                     int64_t step, float grad_scale, void* stream);
 
 #ifdef __cplusplus
 }

@@ -40,7 +40,7 @@ def master_step(master: torch.Tensor, grad_lp: torch.Tensor, m: torch.Tensor, v:
 
 
 def lp_step(p: torch.Tensor, g: torch.Tensor, m: torch.Tensor, v: torch.Tensor, step: int, lr: float, **kw):
-    """AdamW with parameter and both moments stored in p.dtype: fp32 arithmetic, each state rounded once."""
-    dt = p.dtype
+    """AdamW on a low-precision parameter updated in place: fp32 arithmetic, then the parameter is rounded once to
+    p.dtype and the moments once to their own dtype (p.dtype as the reference holds them, or fp32)."""
     p2, m2, v2 = adamw_step(p.float(), g.float(), m.float(), v.float(), step, lr, **kw)
-    return p2.to(dt), m2.to(dt), v2.to(dt)
+    return p2.to(p.dtype), m2.to(m.dtype), v2.to(v.dtype)

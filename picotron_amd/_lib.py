@@ -43,8 +43,8 @@ SIGNATURES = {
     "pico_cross_entropy_fwd": (c_int, [_P, _P, _P, _P, _I64, _I64, _I64, _I64, c_int, _P]),
     "pico_cross_entropy_bwd": (c_int, [_P, _P, _P, _P, _P, _I64, _I64, _I64, _I64, _I64, c_int, _P]),
     "pico_adamw": (c_int, [_P, _P, _P, c_int, _P, _P, _I64] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
-    "pico_adamw_lp": (c_int, [_P, _P, c_int, _P, _P, _I64, c_int] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
-    "pico_adamw_multi": (c_int, [c_int, _P, _P, _P, _P, _P, _P, c_int, c_int] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
+    "pico_adamw_lp": (c_int, [_P, _P, c_int, _P, _P, _I64, c_int, c_int] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
+    "pico_adamw_multi": (c_int, [c_int, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int] + [ctypes.c_float] * 5 + [_I64, ctypes.c_float, _P]),
     "pico_convert_f32": (c_int, [_P, _P] + [_I64] * 7 + [c_int, _P]),
 }
 

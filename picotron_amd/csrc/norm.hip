@@ -179,7 +179,7 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
 // next row: loads and stores retire in one order, so waiting for a prefetched row also waits for the stores
 // of the current one (measured: 3.4 TB/s with the prefetch, 5.2 TB/s -- the rate of a plain copy -- without).  The block's four waves are summed through LDS once at
 // the end and the block writes one row of the partial-sum workspace.
-template <typename T, int NV>
+template <typename T, int NV, bool kRes>
 __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
     const float* __restrict__ rstd, const T* dres, T* dx, float* __restrict__ partial,
@@ -191,7 +191,7 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
   const int nvec = hidden / V;
   const float inv_h = 1.f / static_cast<float>(hidden);
   float dw[NV][V], wv[NV][V];
-  u32x4 xr[NV], dr[NV], rr[NV];  // rr: the residual stream's own gradient, when there is one
+  u32x4 xr[NV], dr[NV], rr[kRes ? NV : 1];  // rr: the residual stream's own gradient (kRes: dres is given)
   float rs;
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
@@ -208,7 +208,7 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
       const int vc = v < nvec ? v : 0;
       xr[j] = *reinterpret_cast<const u32x4*>(x + r * hidden + vc * V);
       dr[j] = *reinterpret_cast<const u32x4*>(dy + r * hidden + vc * V);
-      if (dres) rr[j] = *reinterpret_cast<const u32x4*>(dres + r * hidden + vc * V);
+      if constexpr (kRes) rr[j] = *reinterpret_cast<const u32x4*>(dres + r * hidden + vc * V);
     }
     rs = rstd[r];
   };
@@ -252,7 +252,7 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
         unpack(dr[j], dv);
 #pragma unroll
         for (int e = 0; e < V; ++e) o[e] = r * (dv[e] * wv[j][e] - xv[e] * r * c);
-        if (dres) {  // dx may alias dres: this lane read its part of the row before it writes it
+        if constexpr (kRes) {  // dx may alias dres: this lane read its part of the row before it writes it
           float rv[V];
           unpack(rr[j], rv);
 #pragma unroll
@@ -406,9 +406,14 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
     const int blocks = bwd_blocks(rows, kBwdWaveThreads / kWave);                                      \
     *blocks_out = blocks;                                                                              \
     const size_t lds = static_cast<size_t>(kBwdWaveThreads / kWave - 1) * hidden * sizeof(float);      \
-    hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV>), dim3(blocks), dim3(kBwdWaveThreads), lds, s,  \
-                       static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w),  \
-                       rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
+    if (dres)                                                                                          \
+      hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV, true>), dim3(blocks), dim3(kBwdWaveThreads), lds, s, \
+                         static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), \
+                         rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
+    else                                                                                               \
+      hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV, false>), dim3(blocks), dim3(kBwdWaveThreads), lds, s, \
+                         static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), \
+                         rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
     return PICO_OK;                                                                                    \
   }
   if (nv_wave && static_cast<size_t>(hidden) * 3 * sizeof(float) <= 65536) {

@@ -2,8 +2,9 @@
 //   pico_adamw     fp32 master weights and moments for low-precision parameters: reads the gradient, the master
 //                  weight and both moments, writes the three fp32 states plus the bf16 copy of the parameter that the
 //                  model computes with.  28 bytes per parameter with a bf16 gradient.
-//   pico_adamw_lp  parameter and both moments kept in bf16 and updated in place (what torch.optim.AdamW holds for a
-//                  bf16 model): the arithmetic is fp32 and every state is rounded once.  14 bytes per parameter.
+//   pico_adamw_lp  the bf16 parameter is updated in place, no master copy; the moments are fp32 (22 bytes per
+//                  parameter) or bf16 (what torch.optim.AdamW holds for a bf16 model; 14 bytes).  The arithmetic is
+//                  fp32 and every stored value is rounded once.
 #include "common.h"
 
 namespace pico {
@@ -30,16 +31,16 @@ __device__ __forceinline__ void store8(__bf16* p, const float (&in)[8]) { io<__b
 // The arithmetic follows torch.optim.AdamW's (non-amsgrad) order of operations so that fp32 states match it to
 // rounding: p *= 1 - lr*wd;  m = m + (g - m)*(1 - b1);  v = v*b2 + g*g*(1 - b2);
 // p -= step_size * m / (sqrt(v) / sqrt(bc2) + eps),  step_size = lr / bc1.
-// TS is the type of the three states (the weight that is updated and both moments); param_lp, when given, receives
-// a bf16 copy of the updated weight.
+// TW is the type of the weight that is updated, TM that of both moments; param_lp, when given, receives a bf16 copy
+// of the updated weight.
 struct Hyper {
   float decay, one_minus_b1, b2, one_minus_b2, step_size, inv_sqrt_bc2, eps, grad_scale;
 };
 
-template <typename TS, typename TG>
-__device__ __forceinline__ void adamw_block(__bf16* __restrict__ param_lp, TS* __restrict__ master,
-                                            const TG* __restrict__ grad, TS* __restrict__ exp_avg,
-                                            TS* __restrict__ exp_avg_sq, int64_t n, int64_t block, const Hyper& h) {
+template <typename TW, typename TM, typename TG>
+__device__ __forceinline__ void adamw_block(__bf16* __restrict__ param_lp, TW* __restrict__ master,
+                                            const TG* __restrict__ grad, TM* __restrict__ exp_avg,
+                                            TM* __restrict__ exp_avg_sq, int64_t n, int64_t block, const Hyper& h) {
   const int64_t i0 = (block * kThreads + threadIdx.x) * kPerThread;
   if (i0 >= n) return;
   float g[kPerThread], p[kPerThread], m[kPerThread], v[kPerThread];
@@ -73,19 +74,19 @@ __device__ __forceinline__ void adamw_block(__bf16* __restrict__ param_lp, TS* _
     if (param_lp) io<__bf16>::store(param_lp + i0, p);
   } else {
     for (int e = 0; e < kPerThread && i0 + e < n; ++e) {
-      master[i0 + e] = static_cast<TS>(p[e]);
-      exp_avg[i0 + e] = static_cast<TS>(m[e]);
-      exp_avg_sq[i0 + e] = static_cast<TS>(v[e]);
+      master[i0 + e] = static_cast<TW>(p[e]);
+      exp_avg[i0 + e] = static_cast<TM>(m[e]);
+      exp_avg_sq[i0 + e] = static_cast<TM>(v[e]);
       if (param_lp) param_lp[i0 + e] = static_cast<__bf16>(p[e]);
     }
   }
 }
 
-template <typename TS, typename TG>
-__global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ param_lp, TS* __restrict__ master,
-                                                         const TG* __restrict__ grad, TS* __restrict__ exp_avg,
-                                                         TS* __restrict__ exp_avg_sq, int64_t n, Hyper h) {
-  adamw_block<TS, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, blockIdx.x, h);
+template <typename TW, typename TM, typename TG>
+__global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ param_lp, TW* __restrict__ master,
+                                                         const TG* __restrict__ grad, TM* __restrict__ exp_avg,
+                                                         TM* __restrict__ exp_avg_sq, int64_t n, Hyper h) {
+  adamw_block<TW, TM, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, blockIdx.x, h);
 }
 
 // Many tensors in one launch: the pointers travel in the kernel arguments (no table in device memory to keep alive),
@@ -102,7 +103,7 @@ struct TensorTable {
   int count;
 };
 
-template <typename TS, typename TG>
+template <typename TW, typename TM, typename TG>
 __global__ __launch_bounds__(kThreads) void adamw_multi_kernel(TensorTable t, Hyper h) {
   const unsigned bid = blockIdx.x;
   int lo = 0, hi = t.count;   // block_start[lo] <= bid < block_start[hi]
@@ -110,9 +111,9 @@ __global__ __launch_bounds__(kThreads) void adamw_multi_kernel(TensorTable t, Hy
     const int mid = (lo + hi) >> 1;
     if (bid >= t.block_start[mid]) lo = mid; else hi = mid;
   }
-  adamw_block<TS, TG>(static_cast<__bf16*>(t.param_lp[lo]), static_cast<TS*>(t.weight[lo]),
-                      static_cast<const TG*>(t.grad[lo]), static_cast<TS*>(t.exp_avg[lo]),
-                      static_cast<TS*>(t.exp_avg_sq[lo]), t.n[lo], bid - t.block_start[lo], h);
+  adamw_block<TW, TM, TG>(static_cast<__bf16*>(t.param_lp[lo]), static_cast<TW*>(t.weight[lo]),
+                          static_cast<const TG*>(t.grad[lo]), static_cast<TM*>(t.exp_avg[lo]),
+                          static_cast<TM*>(t.exp_avg_sq[lo]), t.n[lo], bid - t.block_start[lo], h);
 }
 
 }  // namespace
@@ -147,9 +148,9 @@ Hyper make_hyper(float lr, float beta1, float beta2, float eps, float weight_dec
 
 constexpr int64_t kPerBlock = static_cast<int64_t>(kThreads) * kPerThread;
 
-template <typename TS>
-int adamw_launch(const char* who, void* param_lp, TS* master, const void* grad, int grad_dtype, TS* exp_avg,
-                 TS* exp_avg_sq, int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
+template <typename TW, typename TM>
+int adamw_launch(const char* who, void* param_lp, TW* master, const void* grad, int grad_dtype, TM* exp_avg,
+                 TM* exp_avg_sq, int64_t n, float lr, float beta1, float beta2, float eps, float weight_decay,
                  int64_t step, float grad_scale, void* stream) {
   if (int rc = hyper_check(who, grad_dtype, step)) return rc;
   if (n < 0) return fail(PICO_ERR_SHAPE, "%s: n=%lld must be >= 0", who, static_cast<long long>(n));
@@ -162,15 +163,15 @@ int adamw_launch(const char* who, void* param_lp, TS* master, const void* grad, 
   const unsigned grid = static_cast<unsigned>((n + kPerBlock - 1) / kPerBlock);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (grad_dtype == PICO_BF16)
-    hipLaunchKernelGGL((adamw_kernel<TS, __bf16>), dim3(grid), dim3(kThreads), 0, s, static_cast<__bf16*>(param_lp),
+    hipLaunchKernelGGL((adamw_kernel<TW, TM, __bf16>), dim3(grid), dim3(kThreads), 0, s, static_cast<__bf16*>(param_lp),
                        master, static_cast<const __bf16*>(grad), exp_avg, exp_avg_sq, n, h);
   else
-    hipLaunchKernelGGL((adamw_kernel<TS, float>), dim3(grid), dim3(kThreads), 0, s, static_cast<__bf16*>(param_lp),
+    hipLaunchKernelGGL((adamw_kernel<TW, TM, float>), dim3(grid), dim3(kThreads), 0, s, static_cast<__bf16*>(param_lp),
                        master, static_cast<const float*>(grad), exp_avg, exp_avg_sq, n, h);
   return check_launch(who);
 }
 
-template <typename TS>
+template <typename TW, typename TM>
 int adamw_multi_launch(int count, void* const* weights, void* const* param_lps, const void* const* grads,
                        void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int grad_dtype,
                        const Hyper& h, hipStream_t s) {
@@ -194,9 +195,9 @@ int adamw_multi_launch(int count, void* const* weights, void* const* param_lps, 
     if (t.count == 0) return PICO_OK;
     const unsigned grid = t.block_start[t.count];
     if (grad_dtype == PICO_BF16)
-      hipLaunchKernelGGL((adamw_multi_kernel<TS, __bf16>), dim3(grid), dim3(kThreads), 0, s, t, h);
+      hipLaunchKernelGGL((adamw_multi_kernel<TW, TM, __bf16>), dim3(grid), dim3(kThreads), 0, s, t, h);
     else
-      hipLaunchKernelGGL((adamw_multi_kernel<TS, float>), dim3(grid), dim3(kThreads), 0, s, t, h);
+      hipLaunchKernelGGL((adamw_multi_kernel<TW, TM, float>), dim3(grid), dim3(kThreads), 0, s, t, h);
     t.count = 0;
     return check_launch(who);
   };
@@ -220,9 +221,9 @@ int adamw_multi_launch(int count, void* const* weights, void* const* param_lps, 
 }  // namespace
 
 extern "C" int pico_adamw_multi(int count, void* const* weights, void* const* param_lps, const void* const* grads,
-                                void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int state_dtype,
-                                int grad_dtype, float lr, float beta1, float beta2, float eps, float weight_decay,
-                                int64_t step, float grad_scale, void* stream) {
+                                void* const* exp_avgs, void* const* exp_avg_sqs, const int64_t* sizes, int weight_dtype,
+                                int state_dtype, int grad_dtype, float lr, float beta1, float beta2, float eps,
+                                float weight_decay, int64_t step, float grad_scale, void* stream) {
   const char* who = "pico_adamw_multi";
   if (int rc = hyper_check(who, grad_dtype, step)) return rc;
   if (count < 0) return fail(PICO_ERR_SHAPE, "%s: count=%d must be >= 0", who, count);
@@ -231,27 +232,36 @@ extern "C" int pico_adamw_multi(int count, void* const* weights, void* const* pa
     return fail(PICO_ERR_NULL, "%s: the pointer tables and sizes are required", who);
   const Hyper h = make_hyper(lr, beta1, beta2, eps, weight_decay, step, grad_scale);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (state_dtype == PICO_F32)
-    return adamw_multi_launch<float>(count, weights, param_lps, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
-  if (state_dtype == PICO_BF16) {
-    if (param_lps) return fail(PICO_ERR_NULL, "%s: param_lps must be NULL when the state is bf16 (the weight is the parameter)", who);
-    return adamw_multi_launch<__bf16>(count, weights, nullptr, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
+  if (weight_dtype == PICO_F32 && state_dtype == PICO_F32)
+    return adamw_multi_launch<float, float>(count, weights, param_lps, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
+  if (weight_dtype == PICO_BF16 && (state_dtype == PICO_BF16 || state_dtype == PICO_F32)) {
+    if (param_lps) return fail(PICO_ERR_NULL, "%s: param_lps must be NULL when the weights are bf16 (they are the parameters)", who);
+    if (state_dtype == PICO_BF16)
+      return adamw_multi_launch<__bf16, __bf16>(count, weights, nullptr, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
+    return adamw_multi_launch<__bf16, float>(count, weights, nullptr, grads, exp_avgs, exp_avg_sqs, sizes, grad_dtype, h, s);
   }
-  return fail(PICO_ERR_DTYPE, "%s: state dtype code %d not supported", who, state_dtype);
+  return fail(PICO_ERR_DTYPE, "%s: weight dtype code %d with state dtype code %d not supported", who, weight_dtype, state_dtype);
 }
 
 extern "C" int pico_adamw(void* param_lp, float* master, const void* grad, int grad_dtype, float* exp_avg,
                           float* exp_avg_sq, int64_t n, float lr, float beta1, float beta2, float eps,
                           float weight_decay, int64_t step, float grad_scale, void* stream) {
-  return adamw_launch<float>("pico_adamw", param_lp, master, grad, grad_dtype, exp_avg, exp_avg_sq, n, lr, beta1, beta2,
-                             eps, weight_decay, step, grad_scale, stream);
+  return adamw_launch<float, float>("pico_adamw", param_lp, master, grad, grad_dtype, exp_avg, exp_avg_sq, n, lr, beta1,
+                                    beta2, eps, weight_decay, step, grad_scale, stream);
 }
 
 extern "C" int pico_adamw_lp(void* param, const void* grad, int grad_dtype, void* exp_avg, void* exp_avg_sq,
-                             int64_t n, int dtype, float lr, float beta1, float beta2, float eps, float weight_decay,
-                             int64_t step, float grad_scale, void* stream) {
-  if (dtype != PICO_BF16) return fail(PICO_ERR_DTYPE, "pico_adamw_lp: state dtype code %d not supported (bf16 only)", dtype);
-  return adamw_launch<__bf16>("pico_adamw_lp", nullptr, static_cast<__bf16*>(param), grad, grad_dtype,
-                              static_cast<__bf16*>(exp_avg), static_cast<__bf16*>(exp_avg_sq), n, lr, beta1, beta2, eps,
-                              weight_decay, step, grad_scale, stream);
+                             int64_t n, int param_dtype, int state_dtype, float lr, float beta1, float beta2, float eps,
+                             float weight_decay, int64_t step, float grad_scale, void* stream) {
+  if (param_dtype != PICO_BF16)
+    return fail(PICO_ERR_DTYPE, "pico_adamw_lp: parameter dtype code %d not supported (bf16 only)", param_dtype);
+  if (state_dtype == PICO_BF16)
+    return adamw_launch<__bf16, __bf16>("pico_adamw_lp", nullptr, static_cast<__bf16*>(param), grad, grad_dtype,
+                                        static_cast<__bf16*>(exp_avg), static_cast<__bf16*>(exp_avg_sq), n, lr, beta1,
+                                        beta2, eps, weight_decay, step, grad_scale, stream);
+  if (state_dtype == PICO_F32)
+    return adamw_launch<__bf16, float>("pico_adamw_lp", nullptr, static_cast<__bf16*>(param), grad, grad_dtype,
+                                       static_cast<float*>(exp_avg), static_cast<float*>(exp_avg_sq), n, lr, beta1, beta2,
+                                       eps, weight_decay, step, grad_scale, stream);
+  return fail(PICO_ERR_DTYPE, "pico_adamw_lp: state dtype code %d not supported", state_dtype);
 }

@@ -399,40 +399,44 @@ def adamw_(param_lp: Optional[torch.Tensor], master: torch.Tensor, grad: torch.T
 def adamw_lp_(param: torch.Tensor, grad: torch.Tensor, exp_avg: torch.Tensor, exp_avg_sq: torch.Tensor, step: int,
               lr: float, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8, weight_decay: float = 0.01,
               grad_scale: float = 1.0) -> None:
-    """In-place AdamW step on a bf16 parameter with bf16 moments (the state torch.optim.AdamW holds for a bf16
-    model); fp32 arithmetic, one rounding per state.  `step` counts from 1."""
+    """In-place AdamW step on a bf16 parameter (no master copy) with fp32 moments, or with bf16 moments (the state
+    torch.optim.AdamW holds for a bf16 model); fp32 arithmetic, one rounding per stored value.  `step` counts from 1."""
     _dev(param, grad, exp_avg, exp_avg_sq)
     n = param.numel()
-    for t, what in ((param, "param"), (exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
-        if t.dtype != torch.bfloat16 or not t.is_contiguous() or t.numel() != n:
-            raise RuntimeError(f"adamw_lp_: {what} must be a contiguous bf16 tensor of {n} elements")
+    if param.dtype != torch.bfloat16 or not param.is_contiguous():
+        raise RuntimeError("adamw_lp_: param must be a contiguous bf16 tensor")
+    sdt = exp_avg.dtype
+    for t, what in ((exp_avg, "exp_avg"), (exp_avg_sq, "exp_avg_sq")):
+        if t.dtype != sdt or sdt not in _DT or not t.is_contiguous() or t.numel() != n:
+            raise RuntimeError(f"adamw_lp_: {what} must be a contiguous bf16 or fp32 tensor of {n} elements")
     if grad.numel() != n:
         raise RuntimeError("adamw_lp_: grad has the wrong number of elements")
     grad = grad.contiguous()
     check(_lib.lib().pico_adamw_lp(_ptr(param), _ptr(grad), _dt(grad, "grad"), _ptr(exp_avg), _ptr(exp_avg_sq), n,
-                                   _dt(param, "param"), float(lr), float(beta1), float(beta2), float(eps),
+                                   _dt(param, "param"), _DT[sdt], float(lr), float(beta1), float(beta2), float(eps),
                                    float(weight_decay), int(step), float(grad_scale), _stream()))
 
 
 class AdamWMultiPlan:
     """The AdamW step for a fixed list of tensors in as few launches as they fit (48 tensors each).  Weights, moments
     and sizes are checked and their pointer tables built once; a step only fills in the gradients' addresses, so its
-    host cost is a fraction of a millisecond for a few hundred tensors.  All weights and moments share one dtype:
-    fp32 (master weights; `param_lps` optionally lists the bf16 parameters to rewrite, None entries allowed) or bf16
-    (the weights are the parameters; `param_lps` must be None).  The plan keeps the tensors alive."""
+    host cost is a fraction of a millisecond for a few hundred tensors.  All weights share one dtype and both moments
+    of all tensors another: fp32 weights with fp32 moments (master weights; `param_lps` optionally lists the bf16
+    parameters to rewrite, None entries allowed), or bf16 weights (the parameters themselves; `param_lps` must be None)
+    with fp32 or bf16 moments.  The plan keeps the tensors alive."""
 
     def __init__(self, weights, exp_avgs, exp_avg_sqs, param_lps=None):
         count = len(weights)
         if count == 0 or not (len(exp_avgs) == len(exp_avg_sqs) == count) or (param_lps is not None and len(param_lps) != count):
             raise RuntimeError("adamw_multi_: the lists must have one entry per tensor (and at least one)")
-        sdt = weights[0].dtype
+        wdt, sdt = weights[0].dtype, exp_avgs[0].dtype
         for i in range(count):
             w, m, v = weights[i], exp_avgs[i], exp_avg_sqs[i]
             _dev(w, m, v)
             n = w.numel()
-            for t, what in ((w, "weight"), (m, "exp_avg"), (v, "exp_avg_sq")):
-                if t.dtype != sdt or not t.is_contiguous() or t.numel() != n:
-                    raise RuntimeError(f"adamw_multi_: tensor {i}: {what} must be a contiguous {sdt} tensor of {n} elements")
+            for t, dt, what in ((w, wdt, "weight"), (m, sdt, "exp_avg"), (v, sdt, "exp_avg_sq")):
+                if t.dtype != dt or not t.is_contiguous() or t.numel() != n:
+                    raise RuntimeError(f"adamw_multi_: tensor {i}: {what} must be a contiguous {dt} tensor of {n} elements")
             if param_lps is not None and param_lps[i] is not None:
                 lp = param_lps[i]
                 _dev(lp)
@@ -446,7 +450,7 @@ class AdamWMultiPlan:
         self._lp = table(param_lps) if param_lps is not None else None
         self._numel = [w.numel() for w in weights]
         self._sizes = (ctypes.c_int64 * count)(*self._numel)
-        self._state_dt = _dt(weights[0], "weight")
+        self._weight_dt, self._state_dt = _dt(weights[0], "weight"), _dt(exp_avgs[0], "exp_avg")
 
     def step(self, grads, step: int, lr: float, beta1: float = 0.9, beta2: float = 0.999, eps: float = 1e-8,
              weight_decay: float = 0.01, grad_scale: float = 1.0) -> None:
@@ -465,7 +469,7 @@ class AdamWMultiPlan:
                 keep.append(g)
             g_arr[i] = g.data_ptr()
         check(_lib.lib().pico_adamw_multi(self.count, self._w, self._lp, g_arr, self._m, self._v, self._sizes,
-                                          self._state_dt, _dt(grads[0], "grad"), float(lr), float(beta1), float(beta2),
+                                          self._weight_dt, self._state_dt, _dt(grads[0], "grad"), float(lr), float(beta1), float(beta2),
                                           float(eps), float(weight_decay), int(step), float(grad_scale), _stream()))
 
 

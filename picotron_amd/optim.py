@@ -6,8 +6,10 @@ dead code) on the bf16 model and so keeps the optimizer state in the parameter d
 ``master_weights=True`` (default)  fp32 state: a master copy of every parameter plus both moments in three flat
     buffers; ``step()`` reads each bf16 gradient once and rewrites the bf16 parameter from the updated master weight
     in the same kernel (``pico_adamw``) -- no cast passes.  28 bytes of HBM traffic per parameter.
-``master_weights=False``  the reference's layout: the bf16 parameter is updated in place and both moments are bf16
-    (``pico_adamw_lp``); fp32 arithmetic inside the kernel, one rounding per state.  14 bytes per parameter."""
+``master_weights=False``  the bf16 parameter is updated in place (``pico_adamw_lp``); fp32 arithmetic inside the
+    kernel, one rounding per stored value.  ``state_dtype=torch.float32`` keeps both moments in fp32 ("bf16 parameters
+    with fp32 AdamW state", 22 bytes per parameter); ``state_dtype=None`` keeps them in the parameter dtype, which is
+    the reference's own layout (14 bytes per parameter)."""
 from __future__ import annotations
 
 from typing import Iterable
@@ -19,7 +21,7 @@ from . import ops
 
 class FusedAdamW:
     def __init__(self, params: Iterable[torch.nn.Parameter], lr: float = 1e-3, betas=(0.9, 0.999), eps: float = 1e-8,
-                 weight_decay: float = 1e-2, overlap_with_backward: bool = False, master_weights: bool = True):
+                 weight_decay: float = 1e-2, overlap_with_backward: bool = False, master_weights: bool = True, state_dtype=None):
         self.params = [p for p in params if p.requires_grad]
         if not self.params:
             raise ValueError("FusedAdamW: no parameters")
@@ -37,14 +39,19 @@ class FusedAdamW:
             total += (p.numel() + 7) // 8 * 8
         self.master_weights = master_weights
         if master_weights:
+            if state_dtype not in (None, torch.float32):
+                raise RuntimeError("FusedAdamW: master weights come with fp32 moments")
             state_dtype = torch.float32
             self.master = torch.zeros(total, dtype=torch.float32, device=dev)
             for p, off in zip(self.params, self.offsets):
                 self.master[off:off + p.numel()].copy_(p.detach().reshape(-1))
         else:
-            state_dtype = self.params[0].dtype
-            if any(p.dtype != state_dtype for p in self.params):
+            if any(p.dtype != self.params[0].dtype for p in self.params):
                 raise RuntimeError("FusedAdamW(master_weights=False): all parameters must share one dtype")
+            if state_dtype is None:
+                state_dtype = self.params[0].dtype
+            if state_dtype not in (torch.float32, self.params[0].dtype):
+                raise RuntimeError("FusedAdamW: state_dtype must be torch.float32 or the parameter dtype")
             self.master = None
         self.exp_avg = torch.zeros(total, dtype=state_dtype, device=dev)
         self.exp_avg_sq = torch.zeros(total, dtype=state_dtype, device=dev)

@@ -473,26 +473,33 @@ def test_adamw_kernel_against_oracle(ops, device, n, grad_dtype):
 
 
 @pytest.mark.parametrize("n,grad_dtype", [(8 * 1024 + 3, torch.bfloat16), (4096, torch.float32), (5, torch.bfloat16)])
-def test_adamw_lp_kernel_against_oracle(ops, device, n, grad_dtype):
-    """pico_adamw_lp (bf16 parameter and moments updated in place) over four steps against oracle.optim.lp_step fed the
-    kernel's own previous state: both compute in fp32 and round once, so almost every element is identical and the rest
-    are one bf16 rounding step apart (the compiler may contract a multiply-add that the oracle rounds twice)."""
+@pytest.mark.parametrize("moment_dtype", [torch.bfloat16, torch.float32])
+def test_adamw_lp_kernel_against_oracle(ops, device, n, grad_dtype, moment_dtype):
+    """pico_adamw_lp (bf16 parameter updated in place, bf16 or fp32 moments) over four steps against
+    oracle.optim.lp_step fed the kernel's own previous state: both compute in fp32 and round once, so almost every
+    element is identical and the rest are one rounding step apart (the compiler may contract a multiply-add that the
+    oracle rounds twice); fp32 moments agree to a few ulp."""
     from oracle import optim as OO
     g = torch.Generator().manual_seed(13)
     p = torch.randn(n, generator=g).bfloat16()
-    d_p, d_m, d_v = p.to(device), torch.zeros(n, dtype=torch.bfloat16, device=device), torch.zeros(n, dtype=torch.bfloat16, device=device)
+    d_p, d_m, d_v = p.to(device), torch.zeros(n, dtype=moment_dtype, device=device), torch.zeros(n, dtype=moment_dtype, device=device)
     for step in range(1, 5):
         grad = (torch.randn(n, generator=g) * 0.05 * step).to(grad_dtype)
         want = OO.lp_step(d_p.cpu(), grad, d_m.cpu(), d_v.cpu(), step, 2e-3, beta1=0.9, beta2=0.95, eps=1e-8, weight_decay=0.1)
         ops.adamw_lp_(d_p, grad.to(device), d_m, d_v, step, 2e-3, 0.9, 0.95, 1e-8, 0.1)
         for got, w in zip((d_p, d_m, d_v), want):
+            assert got.dtype == w.dtype
             diff = (got.cpu().float() - w.float()).abs()
+            if w.dtype == torch.float32:
+                assert (diff <= 1e-6 * w.abs().max().clamp_min(1e-3)).all()
+                continue
             assert (diff <= w.float().abs() * 2.0 ** -7 + w.float().abs().mean() * 2.0 ** -14).all()
             assert (diff != 0).sum().item() <= max(1, 0.03 * n)
 
 
-@pytest.mark.parametrize("state_dtype", [torch.bfloat16, torch.float32])
-def test_adamw_multi_equals_one_call_per_tensor(ops, device, state_dtype):
+@pytest.mark.parametrize("state_dtype,moment_dtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                                      (torch.float32, torch.float32)])
+def test_adamw_multi_equals_one_call_per_tensor(ops, device, state_dtype, moment_dtype):
     """pico_adamw_multi over 61 tensors (more than one launch's table holds; sizes 0, 1, odd and many blocks) leaves
     every state bit-identical to pico_adamw / pico_adamw_lp called once per tensor."""
     g = torch.Generator().manual_seed(17)
@@ -500,8 +507,8 @@ def test_adamw_multi_equals_one_call_per_tensor(ops, device, state_dtype):
     lp = state_dtype == torch.bfloat16
     def fresh():
         gg = torch.Generator().manual_seed(18)
-        mk = lambda n, pos=False: (torch.rand(n, generator=gg) if pos else torch.randn(n, generator=gg)).to(state_dtype).to(device)
-        return ([mk(n) for n in sizes], [mk(n) for n in sizes], [mk(n, True) for n in sizes],
+        mk = lambda n, dt=state_dtype, pos=False: (torch.rand(n, generator=gg) if pos else torch.randn(n, generator=gg)).to(dt).to(device)
+        return ([mk(n) for n in sizes], [mk(n, moment_dtype) for n in sizes], [mk(n, moment_dtype, True) for n in sizes],
                 [torch.randn(n, generator=gg).bfloat16().to(device) for n in sizes])
     w1, m1, v1, gr = fresh()
     w2, m2, v2, _ = fresh()
@@ -520,6 +527,31 @@ def test_adamw_multi_equals_one_call_per_tensor(ops, device, state_dtype):
             assert torch.equal(lp1[i], lp2[i])
     with pytest.raises(RuntimeError, match="one entry per tensor"):
         ops.adamw_multi_(w1, gr[:-1], m1, v1, *hyper)
+
+
+def test_fused_adamw_with_fp32_moments_and_no_master_copy(device):
+    """FusedAdamW(master_weights=False, state_dtype=fp32): bf16 parameters updated in place, fp32 moments.  The moments
+    follow torch.optim.AdamW run on fp32 copies fed the same gradients (they do not depend on the weights) to fp32
+    accuracy; the parameters follow it to bf16 rounding accumulated over the steps."""
+    from picotron_amd.optim import FusedAdamW
+    torch.manual_seed(9)
+    ps = [torch.nn.Parameter(torch.randn(33, 20, device=device).to(torch.bfloat16)), torch.nn.Parameter(torch.randn(7, device=device).to(torch.bfloat16))]
+    ref = [torch.nn.Parameter(p.detach().float().clone()) for p in ps]
+    opt = FusedAdamW(ps, lr=1e-2, weight_decay=0.02, master_weights=False, state_dtype=torch.float32)
+    ropt = torch.optim.AdamW(ref, lr=1e-2, weight_decay=0.02)
+    assert opt.master is None and opt.exp_avg.dtype == torch.float32
+    for _ in range(3):
+        for p, r in zip(ps, ref):
+            p.grad = torch.randn_like(p)
+            r.grad = p.grad.float()
+        opt.step()
+        ropt.step()
+    for p, r, off in zip(ps, ref, opt.offsets):
+        n = p.numel()
+        st = ropt.state[r]
+        assert maxabs(opt.exp_avg[off:off + n].view_as(p), st["exp_avg"]) <= 1e-6
+        assert maxabs(opt.exp_avg_sq[off:off + n].view_as(p), st["exp_avg_sq"]) <= 1e-6
+        assert maxabs(p.detach().float(), r.detach()) <= 3 * 2 ** -8 * r.detach().abs().max().item()
 
 
 def test_fused_adamw_without_master_weights_follows_torch_fused_adamw(device):
