@@ -52,6 +52,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the extra kernels")
     ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B- and Llama-2-7B-shaped training steps")
+    ap.add_argument("--train-step", choices=["smollm_1p7b", "llama2_7b"], default=None,
+                    help="run only that training step (for a kernel trace of it) and print its figures")
     ap.add_argument("--probe", action="store_true",
                     help="counter probe: a few launches of a plain copy of known size and of each attention kernel "
                          "at the bench shape, nothing else (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
@@ -432,6 +434,9 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     ops._lib.lib()  # fail loudly now if the HIP library is not built
 
+    if args.train_step:
+        print(json.dumps({args.train_step + "_train_step": train_step_extra(torch, args.train_step, steps=4, warmup=2)}))
+        return
     rb = RingBench(torch, ops)
     if args.probe:
         # plain copy of 64 MiB fp32 (read 64 MiB, write 64 MiB) as the scale for the HBM counters
