@@ -96,6 +96,34 @@ def test_configs3_llama2_7b_attention_shape(ops, device):
     assert rel_l2(dq[:, :4], w_dq) <= 1e-2 and rel_l2(dk[:, :4], w_dk) <= 1e-2 and rel_l2(dv[:, :4], w_dv) <= 1e-2
 
 
+@pytest.mark.parametrize("Sq,Sk,q_offset,Hkv", [(2100, 2100, 0, 32), (1790, 2081, 291, 8), (2049, 4100, 2051, 8)])
+def test_head_dim_128_large_launch_ragged_lengths(ops, device, Sq, Sk, q_offset, Hkv):
+    """head_dim 128 with enough workgroups for the large-launch kernels (128-key staged tiles in the forward), at
+    lengths that are multiples of neither the query tile nor the key tile, with the causal diagonal shifted and GQA:
+    forward and backward against an fp32 torch reference on a slice of the heads (first and last kv head)."""
+    Hq, D = 32, 128
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator(device="cpu").manual_seed(5)
+    q = (torch.randn(1, Hq, Sq, D, generator=g)).to(torch.bfloat16).to(device)
+    k = torch.randn(1, Hkv, Sk, D, generator=g).to(torch.bfloat16).to(device)
+    v = torch.randn(1, Hkv, Sk, D, generator=g).to(torch.bfloat16).to(device)
+    do = torch.randn(1, Hq, Sq, D, generator=g).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(q, k, v, scale, True, q_offset)
+    dq, dk, dv = ops.attn_bwd(do, q, k, v, lse, None, scale, True, q_offset, dq_dtype=torch.bfloat16,
+                              dkv_dtype=torch.bfloat16, out=out)
+    rep = Hq // Hkv
+    for kvh in (0, Hkv - 1):
+        qs = slice(kvh * rep, (kvh + 1) * rep)
+        r_o, r_l, r_dq, r_dk, r_dv = ref_attention_fp32(q[:, qs], k[:, kvh:kvh + 1], v[:, kvh:kvh + 1], scale, q_offset, do[:, qs])
+        assert maxabs(out[:, qs], r_o) <= 2e-2 and maxabs(lse[:, qs], r_l) <= 1e-3
+        assert rel_l2(dq[:, qs], r_dq) <= 1e-2
+        assert rel_l2(dk[:, kvh:kvh + 1], r_dk) <= 1e-2 and rel_l2(dv[:, kvh:kvh + 1], r_dv) <= 1e-2
+    # keys that no query may see get exactly zero gradient
+    last_visible = q_offset + Sq - 1
+    if last_visible + 1 < Sk:
+        assert dk[:, :, last_visible + 1:].abs().max().item() == 0.0 and dv[:, :, last_visible + 1:].abs().max().item() == 0.0
+
+
 def test_configs4_long_context_rank7_of_8(ops, device):
     """configs[4]: rank 7 of cp 8 at total seq 32768 -- a 4096-token q chunk over 8 K/V chunks of 4096, GQA 32/8,
     head_dim 128, with RoPE at absolute positions.  Full size on the GPU; checks: RoPE offset == sliced tables (exact),
