@@ -49,6 +49,12 @@ constexpr bool kStreamGrads = PICO_STREAM_GRADS != 0;
 #define PICO_PIPELINE_TRIP 1
 #endif
 constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
+#ifndef PICO_DKDV_STAGES128
+#define PICO_DKDV_STAGES128 1
+#endif
+#ifndef PICO_DKDV_STAGES64
+#define PICO_DKDV_STAGES64 0
+#endif
 
 template <int D>
 struct KvCfg {
@@ -283,6 +289,87 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       // that lets the wave's own phases overlap -- the matrix pipe works on the second sub-block's S / dP while the
       // vector pipe does the first one's softmax, and on the first one's dV / dK during the second one's softmax.
       f32x16 s0, d0, s1, d1;
+      if constexpr (D >= 128 ? PICO_DKDV_STAGES128 != 0 : PICO_DKDV_STAGES64 != 0) {
+      // Four stages; in the middle two, every pair of MFMAs is followed in program order by a share of the OTHER
+      // sub-block's softmax arithmetic and by the LDS reads of a later pair.  A wave issues in order: vector
+      // instructions that merely follow a batch of MFMAs start when the batch has been issued, i.e. when the matrix
+      // pipe is nearly done with it, while an MFMA followed by a few vector instructions keeps both pipes busy
+      // (measured on this GPU with one wave per SIMD: 16 MFMAs then 64 fma + 16 exp take 1.63x the time of the same
+      // work dealt out one MFMA at a time).  The scheduling barriers pin that order slot by slot.  Used at head_dim 128,
+      // whose kernel runs one wave per SIMD (+5 %); at head_dim 64 a second wave fills the gaps already and the extra
+      // live fragments would spill.
+      constexpr int kPairs = D / 16;        // (S, dP) MFMA pairs per sub-block
+      constexpr int kSlots = 2 * (D / 32);  // (dV, dK) MFMA pairs per sub-block
+      auto softmax_part = [&](f32x16& s_acc, f32x16& dp_acc, const f32x4 (&l4)[4], int first, int count) {
+#pragma unroll
+        for (int i = first; i < first + count; ++i) {
+          const float pv = fast_exp2(s_acc[i] * c - l4[i / 4][i % 4]);
+          s_acc[i] = pv;
+          dp_acc[i] = pv * dp_acc[i];
+        }
+      };
+      // stage A: products of sub-block 0
+      products(0, s0, d0);
+      __builtin_amdgcn_sched_barrier(0);
+      // stage B: products of sub-block 1, softmax of sub-block 0 between them
+      {
+        f32x4 l4[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          l4[j] = *reinterpret_cast<const f32x4*>(&sL[8 * j + 4 * h]);
+          const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 + 8 * j + 4 * h]);
+#pragma unroll
+          for (int t = 0; t < 4; ++t) { s1[4 * j + t] = 0.f; d1[4 * j + t] = d4[t]; }
+        }
+        bf16x8 qa[kPairs], da[kPairs];
+        auto fetch = [&](int j) {
+          qa[j] = *reinterpret_cast<const bf16x8*>(&sQ[(32 + n) * LDQ + 16 * j + 8 * h]);
+          da[j] = *reinterpret_cast<const bf16x8*>(&sdO[(32 + n) * LDQ + 16 * j + 8 * h]);
+        };
+        fetch(0);
+        fetch(1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kPairs; ++j) {
+          if (j + 2 < kPairs) fetch(j + 2);
+          s1 = mfma32(qa[j], kf[j], s1);
+          d1 = mfma32(da[j], vf[j], d1);
+          softmax_part(s0, d0, l4, j * (16 / kPairs), 16 / kPairs);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // stage C: dV / dK of sub-block 0, softmax of sub-block 1 between them
+      {
+        f32x4 l4[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) l4[j] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * j + 4 * h]);
+        bf16x8 dof[kSlots], qf[kSlots];
+        auto fetch = [&](int idx) {
+          const int cc = idx / (D / 32), db = idx % (D / 32);
+          const int qr = 16 * cc + 4 * h + (lane % 16) / 4;
+          const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+          dof[idx] = lds_read_tr_pair(&sdO[qr * LDQ + col], LDQ);
+          qf[idx] = lds_read_tr_pair(&sQ[qr * LDQ + col], LDQ);
+        };
+        fetch(0);
+        bf16x8 pf = pack8(s0, 0), dsf = pack8(d0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int idx = 0; idx < kSlots; ++idx) {
+          const int db = idx % (D / 32);
+          if (idx + 1 < kSlots) fetch(idx + 1);
+          dv_acc[db] = mfma32(dof[idx], pf, dv_acc[db]);
+          dk_acc[db] = mfma32(qf[idx], dsf, dk_acc[db]);
+          if (idx + 1 == D / 32) { pf = pack8(s0, 8); dsf = pack8(d0, 8); }
+          softmax_part(s1, d1, l4, idx * (16 / kSlots), 16 / kSlots);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+      // stage D: dV / dK of sub-block 1; the next tile's global loads are issued here, not at the top of the trip:
+      // their registers are free until now
+      if (has_next) prefetch();
+      accumulate(1, s1, d1);
+      } else {
       products(0, s0, d0);
       products(1, s1, d1);
       __builtin_amdgcn_sched_barrier(0);
@@ -292,6 +379,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       if (has_next) prefetch();  // issued here, not at the top of the trip: its registers are free until now
       softmax_grad(1, s1, d1, std::false_type{});
       accumulate(1, s1, d1);
+      }
     } else {
 #pragma unroll
       for (int sb = 0; sb < BM / 32; ++sb) {
