@@ -94,7 +94,9 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   //      else writes before the end of the first trip, a barrier later
   bf16x8 kf[D / 16], vf[D / 16];
   {
-    const int row0 = key0 + 32 * wave;
+    // (the wave index read as a scalar: the buffer windows below are then built in scalar registers; from the
+    // per-lane value the compiler cannot tell that they are the same in all lanes and loops over the lanes' values)
+    const int row0 = key0 + 32 * __builtin_amdgcn_readfirstlane(wave);
     WaveTile<D> kt, vt;
     kt.issue(make_buffer(kbase + static_cast<int64_t>(row0) * a.ks[2], span_bytes(a.Sk - row0, a.ks[2], D)), a.ks[2], lane);
     vt.issue(make_buffer(vbase + static_cast<int64_t>(row0) * a.vs[2], span_bytes(a.Sk - row0, a.vs[2], D)), a.vs[2], lane);
