@@ -61,6 +61,34 @@ def test_argument_checks_run_without_a_gpu():
     assert b"4 GiB" in lib.pico_last_error()
 
 
+def test_argument_checks_of_the_optimizer_and_loss_entries():
+    """Bad dtype codes, negative counts and sizes are refused before anything is launched (no device needed)."""
+    from picotron_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built here")
+    lib = _lib.lib()
+    BF, F32 = _lib.PICO_BF16, _lib.PICO_F32
+    hyper = (1e-3, 0.9, 0.999, 1e-8, 0.01)
+    assert lib.pico_adamw(None, None, None, 99, None, None, 16, *hyper, 1, 1.0, None) == -2          # gradient dtype
+    assert lib.pico_adamw(None, None, None, BF, None, None, 16, *hyper, 0, 1.0, None) == -3          # step counts from 1
+    assert lib.pico_adamw(None, None, None, BF, None, None, 16, *hyper, 1, 1.0, None) == -1          # NULL state
+    assert lib.pico_adamw(None, None, None, BF, None, None, 0, *hyper, 1, 1.0, None) == 0            # nothing to do
+    assert lib.pico_adamw_lp(None, None, BF, None, None, 16, F32, F32, *hyper, 1, 1.0, None) == -2   # parameter must be bf16
+    assert lib.pico_adamw_lp(None, None, BF, None, None, 16, BF, 7, *hyper, 1, 1.0, None) == -2      # state dtype
+    assert lib.pico_adamw_multi(-1, None, None, None, None, None, None, BF, BF, BF, *hyper, 1, 1.0, None) == -3
+    assert lib.pico_adamw_multi(0, None, None, None, None, None, None, BF, BF, BF, *hyper, 1, 1.0, None) == 0
+    assert lib.pico_adamw_multi(2, None, None, None, None, None, None, BF, BF, BF, *hyper, 1, 1.0, None) == -1   # tables
+    one = (ctypes.c_void_p * 1)(None)
+    size = (ctypes.c_int64 * 1)(8)
+    # fp32 weights with bf16 moments is not a layout the library has
+    assert lib.pico_adamw_multi(1, one, None, one, one, one, size, F32, BF, BF, *hyper, 1, 1.0, None) == -2
+    assert b"weight dtype" in lib.pico_last_error()
+    size[0] = -4
+    assert lib.pico_adamw_multi(1, one, None, one, one, one, size, BF, BF, BF, *hyper, 1, 1.0, None) == -3
+    assert lib.pico_rmsnorm_bwd(None, None, None, None, None, None, None, 5, None, 0, 4, 64, BF, None) == -2     # dweight dtype
+    assert lib.pico_cross_entropy_fwd(None, None, None, None, 4, 1000, 1003, -100, BF, None) != 0    # pitch not a multiple of 8
+
+
 def test_cpu_tensors_are_refused_not_computed():
     from picotron_amd import ops
     with pytest.raises(RuntimeError, match="GPU only"):

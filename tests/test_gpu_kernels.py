@@ -645,3 +645,26 @@ def test_fused_adamw_overlapped_with_backward_gives_the_same_update(device):
         results.append([p.detach().float().cpu() for p in params] + [opt.master.cpu()])
     for a, b in zip(*results):
         assert torch.equal(a, b)
+
+
+def test_empty_inputs_are_no_ops(ops, device):
+    """Zero batch, zero queries, zero rows, zero parameters: every entry returns without touching memory."""
+    bf = torch.bfloat16
+    q = torch.zeros(0, 2, 16, 64, dtype=bf, device=device)
+    out, lse = ops.attn_fwd(q, q, q, 0.125, True)
+    assert out.shape == (0, 2, 16, 64) and lse.shape == (0, 2, 16)
+    q0 = torch.zeros(1, 2, 0, 64, dtype=bf, device=device)
+    kv = torch.randn(1, 2, 16, 64, device=device).to(bf)
+    out, lse = ops.attn_fwd(q0, kv, kv, 0.125, False)
+    assert out.numel() == 0 and lse.numel() == 0
+    dq, dk, dv = ops.attn_bwd(q0, q0, kv, kv, lse, lse.clone(), 0.125, False, 0, dq_dtype=bf, dkv_dtype=bf)
+    assert dq.numel() == 0 and dk.abs().max().item() == 0.0 and dv.abs().max().item() == 0.0   # no query: zero gradients
+    cos, sin = OL.get_cos_sin(8, 64, 10000.0)
+    assert ops.rope(torch.zeros(1, 2, 0, 64, dtype=bf, device=device), cos.to(device), sin.to(device)).numel() == 0
+    logits = torch.zeros(0, 64, dtype=bf, device=device)
+    loss_rows, lse_rows = ops.cross_entropy_fwd(logits, torch.zeros(0, dtype=torch.int64, device=device))
+    assert loss_rows.numel() == 0 and lse_rows.numel() == 0
+    e = torch.zeros(0, dtype=bf, device=device)
+    ops.adamw_lp_(e, e, e.clone(), e.clone(), 1, 1e-3)
+    ops.adamw_multi_([e], [e], [e.clone()], [e.clone()], 1, 1e-3)
+    torch.cuda.synchronize()
