@@ -53,7 +53,7 @@ constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 #define PICO_DKDV_STAGES128 1
 #endif
 #ifndef PICO_DKDV_STAGES64
-#define PICO_DKDV_STAGES64 0
+#define PICO_DKDV_STAGES64 1
 #endif
 
 template <int D>
@@ -297,9 +297,10 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       // instructions that merely follow a batch of MFMAs start when the batch has been issued, i.e. when the matrix
       // pipe is nearly done with it, while an MFMA followed by a few vector instructions keeps both pipes busy
       // (measured on this GPU with one wave per SIMD: 16 MFMAs then 64 fma + 16 exp take 1.63x the time of the same
-      // work dealt out one MFMA at a time).  The scheduling barriers pin that order slot by slot.  Used at head_dim 128,
-      // whose kernel runs one wave per SIMD (+5 %); at head_dim 64 a second wave fills the gaps already and the extra
-      // live fragments would spill.
+      // work dealt out one MFMA at a time).  The scheduling barriers pin that order slot by slot (+5 % at head_dim 128,
+      // one wave per SIMD; +2.5 % at head_dim 64, where the second wave of the SIMD fills most gaps already).  The
+      // head_dim 64 kernel has 256 registers: fragments are fetched one pair ahead and lse rows one slot ahead so
+      // that nothing spills.
       constexpr int kPairs = D / 16;        // (S, dP) MFMA pairs per sub-block
       constexpr int kSlots = 2 * (D / 32);  // (dV, dK) MFMA pairs per sub-block
       auto softmax_part = [&](f32x16& s_acc, f32x16& dp_acc, const f32x4 (&l4)[4], int first, int count) {
@@ -315,10 +316,13 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       __builtin_amdgcn_sched_barrier(0);
       // stage B: products of sub-block 1, softmax of sub-block 0 between them
       {
+        // lse rows of sub-block 0 are fetched a slot ahead of the elements that need them (kPer elements per slot)
+        constexpr int kPer = 16 / kPairs;
         f32x4 l4[4];
+        auto lse_row = [&](int r) { l4[r] = *reinterpret_cast<const f32x4*>(&sL[8 * r + 4 * h]); };
+        lse_row(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          l4[j] = *reinterpret_cast<const f32x4*>(&sL[8 * j + 4 * h]);
           const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 + 8 * j + 4 * h]);
 #pragma unroll
           for (int t = 0; t < 4; ++t) { s1[4 * j + t] = 0.f; d1[4 * j + t] = d4[t]; }
@@ -328,23 +332,26 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
           qa[j] = *reinterpret_cast<const bf16x8*>(&sQ[(32 + n) * LDQ + 16 * j + 8 * h]);
           da[j] = *reinterpret_cast<const bf16x8*>(&sdO[(32 + n) * LDQ + 16 * j + 8 * h]);
         };
-        fetch(0);
-        fetch(1);
+        constexpr int kAhead = D >= 128 ? 2 : 1;   // fragment pairs in flight ahead of their MFMAs
+#pragma unroll
+        for (int j = 0; j < kAhead; ++j) fetch(j);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int j = 0; j < kPairs; ++j) {
-          if (j + 2 < kPairs) fetch(j + 2);
+          if (j + kAhead < kPairs) fetch(j + kAhead);
+          if (((j + 1) * kPer) % 4 == 0 && (j + 1) * kPer < 16) lse_row((j + 1) * kPer / 4);
           s1 = mfma32(qa[j], kf[j], s1);
           d1 = mfma32(da[j], vf[j], d1);
-          softmax_part(s0, d0, l4, j * (16 / kPairs), 16 / kPairs);
+          softmax_part(s0, d0, l4, j * kPer, kPer);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
       // stage C: dV / dK of sub-block 0, softmax of sub-block 1 between them
       {
+        constexpr int kPer = 16 / kSlots;
         f32x4 l4[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) l4[j] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * j + 4 * h]);
+        auto lse_row = [&](int r) { l4[r] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * r + 4 * h]); };
+        lse_row(0);
         bf16x8 dof[kSlots], qf[kSlots];
         auto fetch = [&](int idx) {
           const int cc = idx / (D / 32), db = idx % (D / 32);
@@ -363,7 +370,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
           dv_acc[db] = mfma32(dof[idx], pf, dv_acc[db]);
           dk_acc[db] = mfma32(qf[idx], dsf, dk_acc[db]);
           if (idx + 1 == D / 32) { pf = pack8(s0, 8); dsf = pack8(d0, 8); }
-          softmax_part(s1, d1, l4, idx * (16 / kSlots), 16 / kSlots);
+          if (((idx + 1) * kPer) % 4 == 0 && (idx + 1) * kPer < 16) lse_row((idx + 1) * kPer / 4);
+          softmax_part(s1, d1, l4, idx * kPer, kPer);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
