@@ -456,10 +456,14 @@ template <> struct KvKernel<64> { static constexpr auto fn = &attn_bwd_dkdv_kern
 template <> struct KvKernel<128> { static constexpr auto fn = &attn_bwd_dkdv_kernel_d128; };
 
 // =====================================================================================  dQ
-template <int D, int NW, int KT>
+// KS > 1: KS waves share the same 32 queries and each takes one 64-key step of every staged tile (see the forward
+// kernel); their dQ partial sums meet in LDS at the end.
+template <int D, int NW, int KT, int KS = 1>
 struct DqCfg {
   static constexpr int kThreads = 64 * NW;
-  static constexpr int BM = 32 * NW;       // queries per workgroup (32 per wave)
+  static constexpr int kQWaves = NW / KS;
+  static constexpr int BM = 32 * kQWaves;  // queries per workgroup (32 per query wave)
+  static_assert(NW % KS == 0 && (KS == 1 || KT == 64 * KS), "one 64-key step of every staged tile per key-split wave");
   static constexpr int BN = 64;            // keys per compute step
   static constexpr int LDK = D + 8;        // pitch of the K and V tiles
   static constexpr int kVecPerRow = D / 8;
@@ -469,11 +473,14 @@ struct DqCfg {
   static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
   static_assert(NW * WaveTile<D>::kRegionBytes <= kLdsBytes, "the Q / dO fragments pass through the tile buffers");
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
+  static constexpr size_t kExchangeBytes = (D / 32) * 16 * 64 * 4;   // a wave's dQ^T accumulators
+  static_assert(KS == 1 || NW * kExchangeBytes <= kLdsBytes, "the exchange reuses the tile buffers");
 };
 
-template <int D, int NW, int KT, bool kDelta>
-__global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p) {
-  using C = DqCfg<D, NW, KT>;
+// (small workgroups are built for two of them per CU: at most 256 registers per lane)
+template <int D, int NW, int KT, bool kDelta, int KS = 1>
+__global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bwd_dq_kernel(const BwdParams p) {
+  using C = DqCfg<D, NW, KT, KS>;
   constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
@@ -487,6 +494,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
   const int q0 = qtile * BM;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int n = lane % 32, h = lane / 32;
+  const int qw = wave % C::kQWaves, ks = wave / C::kQWaves;   // which queries, which 64-key step of a staged tile
   const float c = a.sm_scale * kLog2e;
 
   const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
@@ -494,12 +502,12 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
 
   // ---- per-lane query: Q and dO fragments (B operands: fetched row-major, turned into fragments through the
   //      wave's piece of LDS; the tile buffers are filled only after the barrier below), lse and delta
-  const int qrow = q0 + wave * 32 + n;
+  const int qrow = q0 + qw * 32 + n;
   const bool qlive = qrow < a.Sq;
   bf16x8 qf[D / 16], dof[D / 16];
   float lse2 = INFINITY, delta = 0.f;
   {
-    const int row0 = q0 + wave * 32;
+    const int row0 = q0 + qw * 32;
     WaveTile<D> qt, dt;
     qt.issue(make_buffer(a.q + b * a.qs[0] + hq * a.qs[1] + static_cast<int64_t>(row0) * a.qs[2],
                          span_bytes(a.Sq - row0, a.qs[2], D)), a.qs[2], lane);
@@ -529,7 +537,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
 #pragma unroll
         for (int e = 0; e < 8; ++e) part += static_cast<float>(dof[s][e]) * static_cast<float>(of[s][e]);
       delta = half_sum(part);
-      if (qlive && h == 0) p.delta_w[gi] = delta;
+      if (qlive && h == 0 && ks == 0) p.delta_w[gi] = delta;
     }
   }
 
@@ -596,7 +604,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
   if (ntiles > 1) load_tile();
   __syncthreads();
 
-  const int blk_q_lo = a.q_offset + q0 + wave * 32;  // position of this wave's first query
+  const int blk_q_lo = a.q_offset + q0 + qw * 32;  // position of this wave's first query
   const int qpos = a.q_offset + qrow;
   for (int t = 0; t < ntiles; ++t) {
     if (t + 1 < ntiles) {
@@ -607,6 +615,7 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     const __bf16* sV = sK + KT * LDK;
 #pragma unroll
     for (int sub = 0; sub < KT / BN; ++sub) {
+      if (KS > 1 && sub != ks) continue;
       const int k0 = t * KT + sub * BN;
       if (k0 >= kv_end) break;
       if (a.causal && k0 > blk_q_lo + 31) continue;  // the wave's whole 32x64 block is in the future
@@ -664,10 +673,34 @@ __global__ __launch_bounds__(64 * NW) void attn_bwd_dq_kernel(const BwdParams p)
     __syncthreads();
   }
 
+  // ---- key split: the partial sums of the waves ks > 0 are added to the wave ks == 0 of the same queries through LDS
+  //      (the loop ended on a barrier: the tile buffers are free; the store pieces used below lie in front of the
+  //      exchange areas of the ks > 0 waves)
+  if constexpr (KS > 1) {
+    float* xo = reinterpret_cast<float*>(smem_raw + wave * C::kExchangeBytes);
+    if (ks > 0) {
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xo[(db * 16 + i) * 64 + lane] = dq[db][i];
+    }
+    __syncthreads();
+    if (ks > 0) return;
+#pragma unroll
+    for (int j = 1; j < KS; ++j) {
+      const float* oo = reinterpret_cast<const float*>(smem_raw + (qw + j * C::kQWaves) * C::kExchangeBytes);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) dq[db][i] += oo[(db * 16 + i) * 64 + lane];
+    }
+    static_assert(kRowRegionBytes <= C::kExchangeBytes, "store pieces lie below the exchange areas read above");
+  }
+
   // ---- epilogue: the wave's 32 dQ rows leave through its piece of LDS as whole lines (the loop ended on a barrier)
   {
     unsigned char* region = smem_raw + wave * kRowRegionBytes;
-    const int row0 = q0 + wave * 32;
+    const int row0 = q0 + qw * 32;
     const int64_t off = b * p.dqs[0] + hq * p.dqs[1] + static_cast<int64_t>(row0) * p.dqs[2];
     if (p.dq_f32)
       wave_store_rows<D, true>(region, dq, a.sm_scale, static_cast<float*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, p.dq_accumulate, false);
@@ -745,22 +778,22 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
   return PICO_OK;
 }
 
-template <int D, int NW, int KT, bool kDelta>
+template <int D, int NW, int KT, bool kDelta, int KS>
 int launch_dq_impl(const BwdParams& p, hipStream_t s) {
-  using C = DqCfg<D, NW, KT>;
+  using C = DqCfg<D, NW, KT, KS>;
   static bool attr_set = false;
   if (!attr_set) {
-    if (int rc = set_lds(&attn_bwd_dq_kernel<D, NW, KT, kDelta>, C::kLdsBytes, "pico_attn_bwd(dq)")) return rc;
+    if (int rc = set_lds(&attn_bwd_dq_kernel<D, NW, KT, kDelta, KS>, C::kLdsBytes, "pico_attn_bwd(dq)")) return rc;
     attr_set = true;
   }
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
-  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, NW, KT, kDelta>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
+  hipLaunchKernelGGL((attn_bwd_dq_kernel<D, NW, KT, kDelta, KS>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
   return PICO_OK;
 }
 
-template <int D, int NW, int KT>
+template <int D, int NW, int KT, int KS = 1>
 int launch_dq(const BwdParams& p, hipStream_t s) {
-  return p.out ? launch_dq_impl<D, NW, KT, true>(p, s) : launch_dq_impl<D, NW, KT, false>(p, s);
+  return p.out ? launch_dq_impl<D, NW, KT, true, KS>(p, s) : launch_dq_impl<D, NW, KT, false, KS>(p, s);
 }
 
 }  // namespace
@@ -857,7 +890,7 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
       auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
       if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
       else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
-      else rc = launch_dq<64, 2, 64>(p, s);
+      else rc = launch_dq<64, 4, 128, 2>(p, s);   // few waves in all: two waves per 32 queries, 64 keys of every 128 each
     } else {
       if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch_dq<128, 8, 64>(p, s);
       else rc = launch_dq<128, 4, 64>(p, s);

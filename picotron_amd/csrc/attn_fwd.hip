@@ -23,10 +23,17 @@ struct FwdParams {
 #ifndef PICO_FWD_KDEPTH
 #define PICO_FWD_KDEPTH (D >= 128 ? 2 : 0)
 #endif
-template <int D, int QB, int NW, int KT>
+// KS > 1 splits the keys of a staged tile over KS waves that share the same queries (NW / KS waves cover the queries):
+// for launches with about one wave per SIMD, where a wave's S -> softmax -> PV chain per key tile is not hidden by
+// anything, this multiplies the waves in flight and divides each chain's length by KS.  The KS partial (m, l, O)
+// states of a query meet in LDS at the end.
+template <int D, int QB, int NW, int KT, int KS = 1>
 struct FwdCfg {
   static constexpr int kThreads = 64 * NW;
-  static constexpr int BM = 32 * QB * NW;  // queries per workgroup
+  static constexpr int kQWaves = NW / KS;        // waves that cover different queries
+  static constexpr int BM = 32 * QB * kQWaves;   // queries per workgroup
+  static_assert(NW % KS == 0 && (KS == 1 || KT == 64 * KS), "one 64-key step of every staged tile per key-split wave");
+  static_assert(KS == 1 || QB == 1, "key split is built for one query block per wave");
   static constexpr int BN = 64;            // keys per compute step
   static constexpr int kKT = KT;           // keys per staged LDS tile (a multiple of BN), double-buffered
   static constexpr int kKDepth = PICO_FWD_KDEPTH;  // K fragments in flight from LDS ahead of the MFMA that uses them (0: compiler's order)
@@ -40,6 +47,9 @@ struct FwdCfg {
   static constexpr int kTileElems = KT * (LDK + LDV);
   static constexpr size_t kLdsBytes = 2 * kTileElems * sizeof(__bf16);
   static_assert(NW * QB * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
+  // exchange of partial states between key-split waves: per wave O^T accumulators (D/32 x 16 registers x 64 lanes) + m + l
+  static constexpr size_t kExchangeBytes = (D / 32) * 16 * 64 * 4 + 2 * 64 * 4;
+  static_assert(KS == 1 || NW * kExchangeBytes <= kLdsBytes, "the exchange reuses the tile buffers");
   static_assert(NW * QB * WaveTile<D>::kRegionBytes <= kLdsBytes, "the Q fragments pass through the tile buffers");
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
@@ -56,12 +66,15 @@ struct FwdCfg {
 #ifndef PICO_FWD_CFG64
 #define PICO_FWD_CFG64 64, 1, 8, PICO_FWD_KT8
 #endif
+#ifndef PICO_FWD_KS
+#define PICO_FWD_KS 2
+#endif
 #ifndef PICO_FWD_ATTR
 #define PICO_FWD_ATTR
 #endif
-template <int D, int QB, int NW, int KT>
+template <int D, int QB, int NW, int KT, int KS = 1>
 __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const FwdParams p) {
-  using C = FwdCfg<D, QB, NW, KT>;
+  using C = FwdCfg<D, QB, NW, KT, KS>;
   constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK, LDV = C::LDV;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   __bf16* smem = reinterpret_cast<__bf16*>(smem_raw);
@@ -79,6 +92,7 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   const int q0 = qtile * BM;
   const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
   const int n = lane % 32, h = lane / 32;
+  const int qw = wave % C::kQWaves, ks = wave / C::kQWaves;   // which queries, which 64-key step of a staged tile
 
   const __bf16* qbase = a.q + b * a.qs[0] + hq * a.qs[1];
   const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
@@ -91,7 +105,7 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   int qrow[QB];
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
-    const int row0 = q0 + (wave * QB + qb) * 32;
+    const int row0 = q0 + (qw * QB + qb) * 32;
     qrow[qb] = row0 + n;
     WaveTile<D> qt;
     qt.issue(make_buffer(qbase + static_cast<int64_t>(row0) * a.qs[2], span_bytes(a.Sq - row0, a.qs[2], D)), a.qs[2], lane);
@@ -111,7 +125,7 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     for (int db = 0; db < D / 32; ++db)
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[qb][db][i] = 0.f;
-    if (p.merge && qrow[qb] < a.Sq) {
+    if (p.merge && ks == 0 && qrow[qb] < a.Sq) {
       // continue from (out, lse) of the earlier blocks: m = lse, l = 1, acc = out
       const float prev = p.lse[lse_row0 + qrow[qb]];
       if (prev != -INFINITY) {
@@ -203,13 +217,14 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
 
 #pragma unroll
     for (int sub = 0; sub < KT / BN; ++sub) {
+      if (KS > 1 && sub != ks) continue;
       const int k0 = t * KT + sub * BN;
       if (k0 >= kv_end) break;
       const __bf16* sKs = sK + sub * BN * LDK;
       const __bf16* sVs = sV + sub * BN * LDV;
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) {
-        const int blk_q_lo = a.q_offset + q0 + (wave * QB + qb) * 32;  // position of the block's first query
+        const int blk_q_lo = a.q_offset + q0 + (qw * QB + qb) * 32;  // position of the block's first query
         if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
         // ---- S^T[key][query] for 64 keys x 32 queries
         f32x16 s_acc[BN / 32];
@@ -315,6 +330,52 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     __syncthreads();  // all waves are done with buffer t&1 (it is refilled in trip t+1) and tile t+1 is visible
   }
 
+  // ---- key split: the waves ks > 0 hand their partial state to the wave ks == 0 of the same queries through LDS
+  //      (the loop ended on a barrier, so the tile buffers are free).  States with different reference maxima m
+  //      combine as O = sum_i 2^(m_i - m) O_i, l = sum_i 2^(m_i - m) l_i with m = max_i m_i.
+  if constexpr (KS > 1) {
+    float* xo = reinterpret_cast<float*>(smem_raw + wave * C::kExchangeBytes);
+    float* xm = xo + (D / 32) * 16 * 64;
+    if (ks > 0) {
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) xo[(db * 16 + i) * 64 + lane] = o[0][db][i];
+      xm[lane] = m_run[0];
+      xm[64 + lane] = l_run[0];
+    }
+    __syncthreads();
+    if (ks > 0) return;
+    float m_all = m_run[0];
+#pragma unroll
+    for (int j = 1; j < KS; ++j) {
+      const float* om = reinterpret_cast<const float*>(smem_raw + (qw + j * C::kQWaves) * C::kExchangeBytes) + (D / 32) * 16 * 64;
+      m_all = fmaxf(m_all, om[lane]);
+    }
+    const float a0 = (m_run[0] == -INFINITY) ? 0.f : fast_exp2(m_run[0] - m_all);
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) o[0][db][i] *= a0;
+    l_run[0] *= a0;
+#pragma unroll
+    for (int j = 1; j < KS; ++j) {
+      const float* oo = reinterpret_cast<const float*>(smem_raw + (qw + j * C::kQWaves) * C::kExchangeBytes);
+      const float* om = oo + (D / 32) * 16 * 64;
+      const float mj = om[lane];
+      const float aj = (mj == -INFINITY) ? 0.f : fast_exp2(mj - m_all);
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) o[0][db][i] += aj * oo[(db * 16 + i) * 64 + lane];
+      l_run[0] += aj * om[64 + lane];
+    }
+    m_run[0] = m_all;
+    // (the rows below leave through the first kQWaves * kRowRegionBytes of LDS, which no exchange area of a ks > 0 wave
+    // overlaps)
+    static_assert(C::kQWaves * kRowRegionBytes <= C::kQWaves * C::kExchangeBytes, "store pieces lie below the exchange areas read above");
+  }
+
   // ---- epilogue: lse per query; the wave's 32 output rows leave through its piece of LDS as whole lines
   //      (the loop ended on a barrier, so the tile buffers are free)
 #pragma unroll
@@ -330,7 +391,7 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
 #pragma unroll
       for (int i = 0; i < 16; ++i) o[qb][db][i] *= inv;
     unsigned char* region = smem_raw + (wave * QB + qb) * kRowRegionBytes;
-    const int row0 = q0 + (wave * QB + qb) * 32;
+    const int row0 = q0 + (qw * QB + qb) * 32;
     const int64_t off = b * a.os[0] + hq * a.os[1] + static_cast<int64_t>(row0) * a.os[2];
     if (p.out_f32)
       wave_store_rows<D, true>(region, o[qb], 1.f, static_cast<float*>(p.out) + off, a.os[2], a.Sq - row0, lane, false, false);
@@ -339,12 +400,12 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   }
 }
 
-template <int D, int QB, int NW, int KT>
+template <int D, int QB, int NW, int KT, int KS = 1>
 int launch(const FwdParams& p, hipStream_t s) {
-  using C = FwdCfg<D, QB, NW, KT>;
+  using C = FwdCfg<D, QB, NW, KT, KS>;
   static bool attr_set = false;
   if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, QB, NW, KT>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, QB, NW, KT, KS>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(C::kLdsBytes)) != hipSuccess)
       return fail(PICO_ERR_LAUNCH, "pico_attn_fwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
     attr_set = true;
@@ -352,7 +413,7 @@ int launch(const FwdParams& p, hipStream_t s) {
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
   FwdParams q = p;
   q.pair_order = p.a.causal && n_qtiles >= 2 && static_cast<int64_t>(p.a.Hq) * p.a.B * n_qtiles <= 512;
-  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW, KT>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, q);
+  hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW, KT, KS>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, q);
   return PICO_OK;
 }
 
@@ -426,7 +487,7 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
     if (groups(256) >= 512) rc = launch<PICO_FWD_CFG64>(p, s);
     else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
-    else rc = launch<64, 1, 2, 64>(p, s);
+    else rc = launch<64, 1, 4, 128, PICO_FWD_KS>(p, s);   // few waves in all: two waves per 32 queries, 64 keys of every 128 each
   } else {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<PICO_FWD_CFG128>(p, s);
