@@ -485,7 +485,8 @@ def main():
     # ---- dominant kernel: the dK/dV launch alone, HIP events on the launching stream.  Its algorithmic work
     #      is 4 of the backward's 5 matrix products (S, dP, dV, dK): 8 FLOPs per (query, key, d) triple.
     dkdv_flops = bwd_flops * 0.8
-    ms_dkdv, _ = graph_time(torch, rb.backward_dkdv_only, max(args.steps // 10, 10), per_graph=10)
+    # (median of three measurements: a single one was once seen 50 % high on an otherwise normal run)
+    ms_dkdv = sorted(graph_time(torch, rb.backward_dkdv_only, max(args.steps // 10, 10), per_graph=10)[0] for _ in range(3))[1]
     dkdv_tflops = dkdv_flops / (ms_dkdv * 1e-3) / 1e12
     roofline = {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel_d64", "achieved": round(dkdv_tflops, 2),
                 "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(dkdv_tflops / MFMA_BF16_PEAK_TFLOPS, 4),
