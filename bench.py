@@ -187,6 +187,20 @@ class RingBench:
         self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
 
 
+def preheat(torch, launch, seconds=0.1, batch=10):
+    """Untimed launches for `seconds` of wall-clock, ending on a synchronize.  The GPU's clocks follow its load with a
+    delay: after an idle stretch (a graph capture, host-side set-up) the first tens of milliseconds of work run about
+    10 % slower than the steady state, so every timed region starts right after one of these.  Returns the launches."""
+    n, t0 = 0, time.perf_counter()
+    while True:
+        for _ in range(batch):
+            launch()
+        torch.cuda.synchronize()
+        n += batch
+        if time.perf_counter() - t0 >= seconds:
+            return n
+
+
 def graph_time(torch, fn, iters, warmup=3, per_graph=1):
     """Records fn() `per_graph` times into a HIP graph and returns (ms per fn() over `iters` replays, graph).
     Each replay is one graph launch, and the GPU idles for about 8 us between two of them; with several
@@ -202,9 +216,7 @@ def graph_time(torch, fn, iters, warmup=3, per_graph=1):
     with torch.cuda.graph(graph):
         for _ in range(per_graph):
             fn()
-    for _ in range(2):
-        graph.replay()
-    torch.cuda.synchronize()
+    preheat(torch, graph.replay, 0.05)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(iters):
@@ -300,7 +312,7 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, adamw="fp32_
     with torch.device("cuda"):
         model = Llama(cfg)
     model = model.to(torch.bfloat16)
-    # one fused pass per parameter tensor (picotron_amd.optim.FusedAdamW over pico_adamw_lp / pico_adamw)
+    # one fused pass over the whole parameter list, up to 48 tensors per launch (picotron_amd.optim.FusedAdamW)
     from picotron_amd.functional import cross_entropy
     from picotron_amd.optim import FusedAdamW
     layouts = {"fp32_moments": (dict(master_weights=False, state_dtype=torch.float32), "bf16 parameters updated in place, fp32 moments"),
@@ -333,8 +345,8 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, adamw="fp32_
     res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
            "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
            "adamw_state": layouts[adamw][1],
-           "note": "attention / RMSNorm / RoPE / SwiGLU / cross-entropy / AdamW on the HIP kernels; embedding, projections "
-                   "and residual adds on torch"}
+           "note": "attention / RMSNorm with the residual adds / RoPE / SwiGLU / cross-entropy / AdamW on the HIP kernels; "
+                   "embedding and projections on torch"}
     del model, opt
     torch.cuda.empty_cache()
     return res
@@ -381,8 +393,38 @@ def long_context_extra(torch, ops, iters=10):
 
     ms_f, _ = graph_time(torch, fused, iters)
     ms_r, _ = graph_time(torch, per_ring_step, iters)
-    return {"flops": flops, "one_launch_per_direction": {"ms": round(ms_f, 3), "TFLOP/s": round(flops / (ms_f * 1e-3) / 1e12, 1)},
-            "one_launch_per_ring_step": {"ms": round(ms_r, 3), "TFLOP/s": round(flops / (ms_r * 1e-3) / 1e12, 1)}}
+    res = {"flops": flops, "one_launch_per_direction": {"ms": round(ms_f, 3), "TFLOP/s": round(flops / (ms_f * 1e-3) / 1e12, 1)},
+           "one_launch_per_ring_step": {"ms": round(ms_r, 3), "TFLOP/s": round(flops / (ms_r * 1e-3) / 1e12, 1)}}
+
+    # RoPE at the rank's absolute positions (r * Sc + arange(Sc)): the q chunk and one K chunk, tables of the whole
+    # sequence, pos_offset instead of sliced tables
+    from picotron_amd.model import get_cos_sin
+    cos, sin = get_cos_sin(W * Sc, D, 10000.0)
+    cos, sin = cos.cuda(), sin.cuda()
+    q_rot = torch.empty_like(q)
+    k_rot = torch.empty_like(k[:, :, :Sc])
+    ms_q, _ = graph_time(torch, lambda: ops.rope(q, cos, sin, pos_offset=r * Sc, out=q_rot), 20, per_graph=10)
+    ms_k, _ = graph_time(torch, lambda: ops.rope(k[:, :, r * Sc:], cos, sin, pos_offset=r * Sc, out=k_rot), 20, per_graph=10)
+    bytes_q, bytes_k = 2 * q.numel() * 2 + Sc * D * 2, 2 * k_rot.numel() * 2 + Sc * D * 2
+    res["rope_at_offset_positions"] = {"q_chunk": {"us": round(ms_q * 1e3, 2), "GB/s": round(bytes_q / (ms_q * 1e-3) / 1e9, 1), "bytes": bytes_q},
+                                       "k_chunk": {"us": round(ms_k * 1e3, 2), "GB/s": round(bytes_k / (ms_k * 1e-3) / 1e9, 1), "bytes": bytes_k},
+                                       "note": "warm (same buffers every launch; 64 MiB and 16 MiB of traffic)"}
+
+    # the reference's layout: K / V expanded to the query heads by repeat_interleave before attention; the kernels then
+    # see 32 kv heads (4 x the K / V traffic and dK / dV of 32 heads)
+    del o32, dq32, dk32, dv32, dk, dv
+    group = Hq // Hkv
+    ke, ve = k.repeat_interleave(group, dim=1), v.repeat_interleave(group, dim=1)
+    dke, dve = torch.empty_like(ke), torch.empty_like(ve)
+
+    def expanded():
+        ops.attn_fwd(q, ke, ve, scale, True, r * Sc, out=out, lse=lse)
+        ops.attn_bwd_preprocess(do, out, delta=delta)
+        ops.attn_bwd(do, q, ke, ve, lse, delta, scale, True, r * Sc, dq, dke, dve)
+
+    ms_e, _ = graph_time(torch, expanded, iters)
+    res["pre_expanded_kv_heads"] = {"ms": round(ms_e, 3), "TFLOP/s": round(flops / (ms_e * 1e-3) / 1e12, 1)}
+    return res
 
 
 def cpu_baseline(host_tensors, W, scale, flops_total):
@@ -403,6 +445,32 @@ def cpu_baseline(host_tensors, W, scale, flops_total):
         out[label] = {"value": round(flops_total / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "s_per_step": round(dt, 3)}
     torch.set_num_threads(cores)
     return out
+
+
+def cpu_long_context_sample(threads):
+    """configs[4] on the CPU oracle, bounded: one dense and one causal chunk-block (4096 x 4096, head_dim 128) for 4 of
+    the 32 query heads (one kv head, expanded as the reference does), forward + backward in fp32; rank 7's 7 dense + 1
+    causal blocks of 32 heads are extrapolated from it (x 8 heads-wise) and labelled as such."""
+    import torch
+    from oracle import ring
+    torch.set_num_threads(threads)
+    Sc, D, Hs = 4096, 128, 4
+    scale = 1.0 / math.sqrt(D)
+    g = torch.Generator().manual_seed(0)
+    q = torch.randn(1, Hs, Sc, D, generator=g) * scale
+    k, v, do = (torch.randn(1, Hs, Sc, D, generator=g) for _ in range(3))
+    secs = {}
+    for name, causal in (("dense", False), ("causal", True)):
+        t0 = time.perf_counter()
+        o, l = ring.block_forward(q, k, v, scale, causal)
+        ring.block_backward(do, q, k, v, o, l, scale, causal)
+        secs[name] = time.perf_counter() - t0
+    rank_s = (7 * secs["dense"] + secs["causal"]) * (32 / Hs)
+    flops = 7.5 * 14 * 32 * Sc * Sc * D
+    return {"s_dense_block_4_heads": round(secs["dense"], 3), "s_causal_block_4_heads": round(secs["causal"], 3),
+            "s_rank7_extrapolated": round(rank_s, 1), "TFLOP/s_extrapolated": round(flops / rank_s / 1e12, 4), "cores": threads,
+            "what": "configs[4]: one dense + one causal 4096x4096 block of 4 query heads on the CPU oracle (fp32), "
+                    "extrapolated to rank 7's 7 dense + 1 causal blocks of 32 heads"}
 
 
 def cpu_configs0_step(threads):
@@ -455,7 +523,8 @@ def main():
     fwd_flops, bwd_flops = rb.flops()
     total_flops = fwd_flops + bwd_flops
 
-    # ---- warm-up (eager), then the timed K replays of the recorded step
+    # ---- W warm-up steps, then EXACTLY K timed steps, twice: as replays of a HIP graph of the step and as plain stream
+    #      launches; each timed region follows 100 ms of the same launches untimed (see preheat).  `value` is the faster.
     for _ in range(max(args.warmup, 1)):
         rb.step_batched()
     torch.cuda.synchronize()
@@ -472,14 +541,21 @@ def main():
     with torch.cuda.graph(graph):
         for _ in range(per_graph):
             rb.step_batched()
-    graph.replay()
-    torch.cuda.synchronize()
+    preheat_steps = preheat(torch, graph.replay, 0.1, batch=2) * per_graph
     t0 = time.perf_counter()
     for _ in range(args.steps // per_graph):
         graph.replay()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
+    ms_graph = (t1 - t0) * 1e3 / args.steps
+    preheat_steps = max(preheat_steps, preheat(torch, rb.step_batched, 0.1, batch=50))
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        rb.step_batched()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_eager = (t1 - t0) * 1e3 / args.steps
+    ms_per_step = min(ms_graph, ms_eager)
     value = total_flops / (ms_per_step * 1e-3) / 1e12
 
     # ---- dominant kernel: the dK/dV launch alone, HIP events on the launching stream.  Its algorithmic work
@@ -512,11 +588,6 @@ def main():
                                       "flops": r3_flops}
         ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
         extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4)}
-        t0 = time.perf_counter()
-        for _ in range(20):
-            rb.step_batched()
-        torch.cuda.synchronize()
-        extras["eager_ms_per_step"] = round((time.perf_counter() - t0) * 1e3 / 20, 4)
         extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
         extras["configs4_long_context_rank7_of_8"] = long_context_extra(torch, ops)
         if not args.no_train:
@@ -531,7 +602,9 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "configs[1]: causal ring attention fwd+bwd, B4 H32 S1024 D64, cp_size 4, the ring steps of all "
                                "4 ranks on one GPU (ranks batched into one launch per direction)",
-                   "global_batch": 4, "seq_len": 1024, "flops_per_step": total_flops, "steps_per_graph_launch": per_graph},
+                   "global_batch": 4, "seq_len": 1024, "flops_per_step": total_flops, "launch": "stream launches" if ms_eager <= ms_graph else "hip graph replays",
+                   "ms_per_step_stream_launches": round(ms_eager, 4), "ms_per_step_graph_replays": round(ms_graph, 4),
+                   "steps_per_graph_launch": per_graph, "untimed_preheat_steps": preheat_steps},
         "frac_of_mfma_peak": round(value / MFMA_BF16_PEAK_TFLOPS, 4),
         "roofline": roofline,
     }
@@ -545,6 +618,7 @@ def main():
         line["cpu_baseline"]["configs0_step"] = {"tokens_per_s_all_threads": round(512 / c0_all, 1), "s_per_step_all_threads": round(c0_all, 3),
                                                  "tokens_per_s_one_thread": round(512 / c0_one, 1), "s_per_step_one_thread": round(c0_one, 3),
                                                  "what": "configs[0]: 2-layer SmolLM-135M shape, fp32, B2 S256, full training step on the CPU oracle"}
+        line["cpu_baseline"]["configs4_sample"] = cpu_long_context_sample(main_leg["cores"])
     if extras:
         line["extras"] = extras
     print(json.dumps(line))
