@@ -124,6 +124,40 @@ def test_head_dim_128_large_launch_ragged_lengths(ops, device, Sq, Sk, q_offset,
         assert dk[:, :, last_visible + 1:].abs().max().item() == 0.0 and dv[:, :, last_visible + 1:].abs().max().item() == 0.0
 
 
+@pytest.mark.parametrize("B,Hkv,Sq,Sk,q_offset,causal", [
+    (4, 32, 1024, 1024, 0, True),      # configs[1] with the four ranks in one launch: the 8-wave kernels
+    (4, 8, 1000, 1000, 0, True),       # 8-wave kernels, ragged, GQA
+    (4, 8, 777, 1203, 0, False),       # 8-wave kernels, dense, rectangular
+    (2, 32, 1024, 1024, 0, True),      # half the batch: the 4-wave kernels without key split
+    (2, 8, 1000, 1290, 290, True),     # 4-wave kernels, ragged, shifted diagonal, GQA
+    (1, 8, 1000, 1290, 290, True),     # key-split kernels on the same lengths
+])
+def test_head_dim_64_every_launch_size_class(ops, device, B, Hkv, Sq, Sk, q_offset, causal):
+    """head_dim 64 at 32 query heads: the library picks 8-wave, 4-wave or key-split workgroups by the number of
+    workgroups a launch has; each class is run here at full and at ragged lengths (forward and backward) and checked
+    against an fp32 torch reference on the first batch entry's first and last GQA group and on the last batch entry."""
+    Hq, D = 32, 64
+    scale = 1 / math.sqrt(D)
+    g = torch.Generator(device="cpu").manual_seed(9)
+    q = torch.randn(B, Hq, Sq, D, generator=g).to(torch.bfloat16).to(device)
+    k = torch.randn(B, Hkv, Sk, D, generator=g).to(torch.bfloat16).to(device)
+    v = torch.randn(B, Hkv, Sk, D, generator=g).to(torch.bfloat16).to(device)
+    do = torch.randn(B, Hq, Sq, D, generator=g).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(q, k, v, scale, causal, q_offset)
+    dq, dk, dv = ops.attn_bwd(do, q, k, v, lse, None, scale, causal, q_offset, dq_dtype=torch.bfloat16,
+                              dkv_dtype=torch.bfloat16, out=out)
+    rep = Hq // Hkv
+    off = q_offset if causal else Sk          # a diagonal past the last key = no mask
+    for b, kvh in ((0, 0), (0, Hkv - 1), (B - 1, Hkv // 2)):
+        bs, qs, ks = slice(b, b + 1), slice(kvh * rep, (kvh + 1) * rep), slice(kvh, kvh + 1)
+        r_o, r_l, r_dq, r_dk, r_dv = ref_attention_fp32(q[bs, qs], k[bs, ks], v[bs, ks], scale, off, do[bs, qs])
+        assert maxabs(out[bs, qs], r_o) <= 2e-2 and maxabs(lse[bs, qs], r_l) <= 1e-3
+        assert rel_l2(dq[bs, qs], r_dq) <= 1e-2
+        assert rel_l2(dk[bs, ks], r_dk) <= 1e-2 and rel_l2(dv[bs, ks], r_dv) <= 1e-2
+    if causal and q_offset + Sq < Sk:
+        assert dk[:, :, q_offset + Sq:].abs().max().item() == 0.0 and dv[:, :, q_offset + Sq:].abs().max().item() == 0.0
+
+
 def test_configs4_long_context_rank7_of_8(ops, device):
     """configs[4]: rank 7 of cp 8 at total seq 32768 -- a 4096-token q chunk over 8 K/V chunks of 4096, GQA 32/8,
     head_dim 128, with RoPE at absolute positions.  Full size on the GPU; checks: RoPE offset == sliced tables (exact),
