@@ -55,6 +55,11 @@ constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 #ifndef PICO_DKDV_STAGES64
 #define PICO_DKDV_STAGES64 1
 #endif
+// Wave priority in the two middle stages of a dK/dV trip (those that mix MFMAs with softmax arithmetic): raised, so
+// that of the two waves of a SIMD the one with vector work to hide issues first (-1.5 % at head_dim 64)
+#ifndef PICO_DKDV_PRIO
+#define PICO_DKDV_PRIO 1
+#endif
 
 template <int D>
 struct KvCfg {
@@ -314,6 +319,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       // stage A: products of sub-block 0
       products(0, s0, d0);
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PICO_DKDV_PRIO != 0) __builtin_amdgcn_s_setprio(PICO_DKDV_PRIO);
       // stage B: products of sub-block 1, softmax of sub-block 0 between them
       {
         // lse rows of sub-block 0 are fetched a slot ahead of the elements that need them (kPer elements per slot)
@@ -377,6 +383,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
       // stage D: dV / dK of sub-block 1; the next tile's global loads are issued here, not at the top of the trip:
       // their registers are free until now
+      if constexpr (PICO_DKDV_PRIO != 0) __builtin_amdgcn_s_setprio(0);
       if (has_next) prefetch();
       accumulate(1, s1, d1);
       } else {
