@@ -300,14 +300,14 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, adamw="fp32_
     import torch.nn.functional as F
 
     import picotron_amd.process_group_manager as pgm
-    from oracle.model import llama2_7b, smollm_1p7b, synthetic_batch
     from picotron_amd.model import Llama
-    from picotron_amd.utils import MI355X_BF16_DENSE_FLOPS, flops_per_token, get_num_params
+    from picotron_amd.utils import (MI355X_BF16_DENSE_FLOPS, flops_per_token, get_num_params, llama2_7b_shape,
+                                    smollm_1p7b_shape, synthetic_tokens)
 
     pgm.setup_process_group_manager(1, 1, 1, 1)
     os.environ["CONTEXT_PARALLEL"] = "0"
     mbs, seq = (4, 1024) if which == "smollm_1p7b" else (1, 4096)
-    cfg = smollm_1p7b(seq) if which == "smollm_1p7b" else llama2_7b(seq)
+    cfg = smollm_1p7b_shape(seq) if which == "smollm_1p7b" else llama2_7b_shape(seq)
     torch.manual_seed(42)
     with torch.device("cuda"):
         model = Llama(cfg)
@@ -320,7 +320,7 @@ def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, adamw="fp32_
                "reference": (dict(master_weights=False), "bf16 moments, bf16 parameter updated in place (the reference's layout)")}
     opt = FusedAdamW(model.parameters(), lr=3e-4, overlap_with_backward=os.getenv("PICO_BENCH_OVERLAP", "0") == "1",
                      **layouts[adamw][0])
-    ids, tgt = synthetic_batch(cfg.vocab_size, mbs, seq, seed=0)
+    ids, tgt = synthetic_tokens(cfg.vocab_size, mbs, seq, seed=0)
     ids, tgt = ids.cuda(), tgt.cuda()
 
     def step():

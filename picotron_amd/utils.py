@@ -3,6 +3,7 @@ MFU formula (:43-49) with MI355X's dense bf16 peak in place of the H100 constant
 from __future__ import annotations
 
 import random
+from dataclasses import dataclass
 
 import numpy as np
 import torch
@@ -38,3 +39,34 @@ def get_mfu(tokens_per_second, num_params, model_config, theoretical_flops=MI355
 
 def get_num_params(model):
     return sum(p.numel() for p in model.parameters())
+
+
+@dataclass
+class ModelShape:
+    """The fields of a Hugging Face Llama config that ``model.Llama`` reads (the reference builds its config with
+    ``AutoConfig.from_pretrained`` and overrides these, ``train.py:154-162``); max_position_embeddings = seq_length."""
+    hidden_size: int
+    num_attention_heads: int
+    num_key_value_heads: int
+    intermediate_size: int
+    vocab_size: int
+    num_hidden_layers: int
+    max_position_embeddings: int
+    rms_norm_eps: float = 1e-5
+    rope_theta: float = 10000.0
+
+
+def smollm_1p7b_shape(seq_length=1024):
+    return ModelShape(2048, 32, 32, 8192, 49152, 24, seq_length)
+
+
+def llama2_7b_shape(seq_length=4096):
+    return ModelShape(4096, 32, 32, 11008, 32000, 32, seq_length)
+
+
+def synthetic_tokens(vocab_size, batch, seq_length, seed):
+    """Token ids uniform over the vocabulary; the targets are the ids shifted by one: seq_length + 1 tokens are drawn
+    per sample and split, as the reference's collate function does (``data.py:102-116``)."""
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(0, vocab_size, (batch, seq_length + 1), generator=g)
+    return ids[:, :-1].contiguous(), ids[:, 1:].contiguous()
