@@ -17,8 +17,12 @@ Parity status of each oracle function (what pins it, see ``tests/test_oracle_*.p
 * ``layers.apply_rotary_pos_emb`` pinned: transformers' ``apply_rotary_pos_emb``; rotation invariants
 * ``layers.rmsnorm*``         pinned: transformers' ``LlamaRMSNorm``, ``F.rms_norm``, autograd
 * ``layers.swiglu*``          pinned: ``F.silu`` (library), autograd
-* ``model.TinyLlama`` step    parity unpinned by any reference fixture (the reference's tests hold none for
-                              this path); it is a composition of the pinned pieces + torch Linear/CE/AdamW.
+* ``layers.cross_entropy*``   pinned: ``F.cross_entropy`` (library), autograd
+* ``optim.adamw_step`` / ``master_step`` pinned: ``torch.optim.AdamW`` step by step
+* ``optim.lp_step``           pinned: torch's fused AdamW on bf16 parameters (rounding points of the stored values)
+* ``model.OracleLlama`` / ``model.train_step``  pinned: transformers' ``LlamaForCausalLM`` with the same weights (logits,
+                              loss, every gradient, one AdamW step), MHA and GQA, with and without the ring
+                              (``tests/test_oracle_model.py``)
 
 The reference ships no golden vectors for any of these functions.
 """
