@@ -134,3 +134,46 @@ def test_local_ring_kv_and_grad_mailbox_on_cpu():
     assert torch.equal(b, torch.full((2,), 12.0))
     assert mgr.cp_ring.deposited[(0, 0)] == {0, 1}
     pgm.setup_process_group_manager(1, 1, 1, 1)
+
+
+C_PROGRAM = r"""
+#include <stdio.h>
+#include <string.h>
+#include "picotron_amd.h"
+int main(void) {
+  pico_attn_desc d;
+  memset(&d, 0, sizeof d);
+  d.B = 1; d.Hq = 2; d.Hkv = 2; d.Sq = 8; d.Sk = 8; d.D = 48;   /* head_dim 48 is not supported */
+  d.sm_scale = 0.125f;
+  int rc = pico_attn_fwd(&d, (void*)16, (void*)16, (void*)16, (void*)16, (float*)16, PICO_BF16, 0, NULL);
+  printf("%s|%d|%s\n", pico_version(), rc, pico_last_error());
+  return rc == PICO_ERR_SHAPE ? 0 : 1;
+}
+"""
+
+
+def test_header_is_plain_c_and_a_c_program_links_against_the_library(tmp_path):
+    """include/picotron_amd.h compiles as C99 with -pedantic, and a C program built with gcc calls the library through
+    it (an argument check that returns before any launch, so no GPU is needed)."""
+    import shutil
+    import subprocess
+    from picotron_amd import _lib
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    inc = os.path.join(ROOT, "include")
+    unit = tmp_path / "unit.c"
+    unit.write_text('#include "picotron_amd.h"\nint main(void) { return 0; }\n')
+    subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-I", inc, str(unit)], check=True)
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("library not built here (python -m picotron_amd.build)")
+    prog = tmp_path / "prog.c"
+    prog.write_text(C_PROGRAM)
+    exe = tmp_path / "prog"
+    libdir = os.path.dirname(_lib.LIB_PATH)
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Werror", "-I", inc, str(prog), "-o", str(exe), "-L", libdir, "-lpicotron_amd",
+                    "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"], check=True)
+    res = subprocess.run([str(exe)], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0, res.stdout + res.stderr
+    version, rc, message = res.stdout.strip().split("|", 2)
+    assert version.startswith("picotron_amd") and int(rc) == -3 and "head_dim" in message
