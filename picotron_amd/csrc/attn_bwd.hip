@@ -57,6 +57,12 @@ constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 #endif
 // Wave priority in the two middle stages of a dK/dV trip (those that mix MFMAs with softmax arithmetic): raised, so
 // that of the two waves of a SIMD the one with vector work to hide issues first (-1.5 % at head_dim 64)
+#ifndef PICO_DKDV_LDQPAD
+#define PICO_DKDV_LDQPAD 32
+#endif
+#ifndef PICO_DKDV_SKEW
+#define PICO_DKDV_SKEW 8
+#endif
 #ifndef PICO_DKDV_PRIO
 #define PICO_DKDV_PRIO 1
 #endif
@@ -67,10 +73,20 @@ struct KvCfg {
   static constexpr int kThreads = 64 * NW;
   static constexpr int BN = 32 * NW;  // keys per workgroup
   static constexpr int BM = 64;       // queries per trip
-  static constexpr int LDQ = D + 8;   // pitch of the Q and dO tiles
+  // Q and dO tiles: rows of D elements at a pitch of LDQ elements, plus kSkew elements after every 4 rows.  Every
+  // tile is read both by rows (16 bytes per lane, 32 consecutive rows per instruction) and transposed (8 bytes per
+  // lane: 4 rows x 32 bytes per 16 lanes, rows 4 apart for the two wave halves).  An LDS instruction takes as many
+  // cycles as its busiest bank (64 banks of 4 bytes) has requests.  With the pitch = 16 (mod 32) words the 16-word
+  // pieces of 4 consecutive rows tile the banks (transposed reads at their minimum of 2 requests per bank; at a pitch
+  // of D + 8 they take 3-4), and the 4-word skew per 4 rows spreads 16 consecutive rows over all multiples of 4 words
+  // (row reads at their minimum of 4).
+  static constexpr int LDQ = D + PICO_DKDV_LDQPAD;
+  static constexpr int kSkew = PICO_DKDV_SKEW;
+  static constexpr int kTileElems = BM * LDQ + kSkew * (BM / 4);       // one tile
+  static constexpr int kTrStep = 8 * LDQ + 2 * kSkew;                  // 8 rows further down
   static constexpr int kVecPerRow = D / 8;
   static constexpr int kQLoads = BM * kVecPerRow / kThreads;
-  static constexpr int kBufElems = 2 * BM * LDQ;                       // Q + dO tile of one stage (bf16)
+  static constexpr int kBufElems = 2 * kTileElems;                     // Q + dO tile of one stage (bf16)
   static constexpr size_t kBufBytes = kBufElems * sizeof(__bf16) + 2 * BM * sizeof(float);
   static constexpr size_t kLdsBytes = 2 * kBufBytes;                   // double-buffered
   static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
@@ -82,6 +98,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   using C = KvCfg<D>;
   constexpr int BM = C::BM, BN = C::BN, LDQ = C::LDQ;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  auto tile_row = [](int r) { return r * C::LDQ + C::kSkew * (r >> 2); };   // element offset of a tile row
 
   const AttnParams& a = p.a;
   const int hkv = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
@@ -185,15 +202,15 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   };
   auto stage = [&](int buf) {  // the prefetched tile (still under the cursor) goes to LDS buffer `buf`
     __bf16* sQ = reinterpret_cast<__bf16*>(smem_raw + buf * C::kBufBytes);
-    __bf16* sdO = sQ + BM * LDQ;
-    float* sL = reinterpret_cast<float*>(sdO + BM * LDQ);
+    __bf16* sdO = sQ + C::kTileElems;
+    float* sL = reinterpret_cast<float*>(sdO + C::kTileElems);
     float* sDelta = sL + BM;
 #pragma unroll
     for (int i = 0; i < C::kQLoads; ++i) {
       const int idx = tid + i * C::kThreads;
       const int r = idx / C::kVecPerRow, cv = idx % C::kVecPerRow;
-      *reinterpret_cast<u32x4*>(&sQ[r * LDQ + cv * 8]) = qreg[i];
-      *reinterpret_cast<u32x4*>(&sdO[r * LDQ + cv * 8]) = doreg[i];
+      *reinterpret_cast<u32x4*>(&sQ[tile_row(r) + cv * 8]) = qreg[i];
+      *reinterpret_cast<u32x4*>(&sdO[tile_row(r) + cv * 8]) = doreg[i];
     }
     if (tid < BM) {
       // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
@@ -225,8 +242,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     if (has_next) advance();
     const int q0 = tile * BM;
     const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + buf_off);
-    const __bf16* sdO = sQ + BM * LDQ;
-    const float* sL = reinterpret_cast<const float*>(sdO + BM * LDQ);
+    const __bf16* sdO = sQ + C::kTileElems;
+    const float* sL = reinterpret_cast<const float*>(sdO + C::kTileElems);
     const float* sDelta = sL + BM;
 
     // The three phases of a 32-query sub-block.
@@ -241,8 +258,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
 #pragma unroll
       for (int s = 0; s < D / 16; ++s) {
-        const bf16x8 qa = *reinterpret_cast<const bf16x8*>(&sQ[(32 * sb + n) * LDQ + 16 * s + 8 * h]);
-        const bf16x8 da = *reinterpret_cast<const bf16x8*>(&sdO[(32 * sb + n) * LDQ + 16 * s + 8 * h]);
+        const bf16x8 qa = *reinterpret_cast<const bf16x8*>(&sQ[tile_row(32 * sb + n) + 16 * s + 8 * h]);
+        const bf16x8 da = *reinterpret_cast<const bf16x8*>(&sdO[tile_row(32 * sb + n) + 16 * s + 8 * h]);
         s_acc = mfma32(qa, kf[s], s_acc);
         dp_acc = mfma32(da, vf[s], dp_acc);
       }
@@ -281,8 +298,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 #pragma unroll
         for (int db = 0; db < D / 32; ++db) {
           const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
-          const bf16x8 dof = lds_read_tr_pair(&sdO[qr * LDQ + col], LDQ);
-          const bf16x8 qf = lds_read_tr_pair(&sQ[qr * LDQ + col], LDQ);
+          const bf16x8 dof = lds_read_tr_pair_step(&sdO[tile_row(qr) + col], C::kTrStep);
+          const bf16x8 qf = lds_read_tr_pair_step(&sQ[tile_row(qr) + col], C::kTrStep);
           dv_acc[db] = mfma32(dof, pf, dv_acc[db]);
           dk_acc[db] = mfma32(qf, dsf, dk_acc[db]);
         }
@@ -335,8 +352,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
         }
         bf16x8 qa[kPairs], da[kPairs];
         auto fetch = [&](int j) {
-          qa[j] = *reinterpret_cast<const bf16x8*>(&sQ[(32 + n) * LDQ + 16 * j + 8 * h]);
-          da[j] = *reinterpret_cast<const bf16x8*>(&sdO[(32 + n) * LDQ + 16 * j + 8 * h]);
+          qa[j] = *reinterpret_cast<const bf16x8*>(&sQ[tile_row(32 + n) + 16 * j + 8 * h]);
+          da[j] = *reinterpret_cast<const bf16x8*>(&sdO[tile_row(32 + n) + 16 * j + 8 * h]);
         };
         constexpr int kAhead = D >= 128 ? 2 : 1;   // fragment pairs in flight ahead of their MFMAs
 #pragma unroll
@@ -363,8 +380,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
           const int cc = idx / (D / 32), db = idx % (D / 32);
           const int qr = 16 * cc + 4 * h + (lane % 16) / 4;
           const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
-          dof[idx] = lds_read_tr_pair(&sdO[qr * LDQ + col], LDQ);
-          qf[idx] = lds_read_tr_pair(&sQ[qr * LDQ + col], LDQ);
+          dof[idx] = lds_read_tr_pair_step(&sdO[tile_row(qr) + col], C::kTrStep);
+          qf[idx] = lds_read_tr_pair_step(&sQ[tile_row(qr) + col], C::kTrStep);
         };
         fetch(0);
         bf16x8 pf = pack8(s0, 0), dsf = pack8(d0, 0);

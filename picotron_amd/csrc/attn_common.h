@@ -44,6 +44,15 @@ __device__ __forceinline__ bf16x8 lds_read_tr_pair(const __bf16* p, int ld) {
   return __builtin_bit_cast(bf16x8, v);
 }
 
+// the same with the second read `step` elements after the first (tiles whose rows are not evenly spaced)
+__device__ __forceinline__ bf16x8 lds_read_tr_pair_step(const __bf16* p, int step) {
+  s16x4 lo = lds_read_tr(p);
+  s16x4 hi = lds_read_tr(p + step);
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(bf16x8, v);
+}
+
 // s_waitcnt immediate for "vmcnt(0)" with the other counters left at their maxima (gfx9 encoding:
 // vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14])
 constexpr int kWaitVmcnt0 = 0x0F70;
