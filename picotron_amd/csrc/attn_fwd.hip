@@ -38,12 +38,11 @@ struct FwdCfg {
   static constexpr int kKT = KT;           // keys per staged LDS tile (a multiple of BN), double-buffered
   static constexpr int kKDepth = PICO_FWD_KDEPTH;  // K fragments in flight from LDS ahead of the MFMA that uses them (0: compiler's order)
   static constexpr int LDK = D + 8;        // K tile pitch: 16-byte row reads hit distinct banks
-#ifndef PICO_FWD_LDVPAD
-#define PICO_FWD_LDVPAD 32
-#endif
-  // V tile pitch for the 4-row transposing reads: 16 (mod 32) words, so that the 16-word pieces of 4 consecutive rows
-  // tile the 64 LDS banks (2 requests per bank, the minimum for an 8-byte read; a pitch of D + 8 gives 3-4)
-  static constexpr int LDV = D + PICO_FWD_LDVPAD;
+  // V tile pitch for the 4-row transposing reads.  At head_dim 128: 16 (mod 32) words, so that the 16-word pieces of 4
+  // consecutive rows tile the 64 LDS banks (2 requests per bank, the minimum for an 8-byte read; a pitch of D + 8 gives
+  // 3-4): -3 %.  At head_dim 64 the kernel's time does not depend on it, and the smaller tile lets two key-split
+  // workgroups (128 staged keys each) share a CU.
+  static constexpr int LDV = D + (D >= 128 ? 32 : 8);
   static constexpr int kVecPerRow = D / 8;
   static constexpr int kLoads = KT * kVecPerRow / kThreads;  // 16-byte loads per thread per tensor
   static constexpr int kTileElems = KT * (LDK + LDV);
