@@ -216,7 +216,7 @@ def graph_time(torch, fn, iters, warmup=3, per_graph=1):
     with torch.cuda.graph(graph):
         for _ in range(per_graph):
             fn()
-    preheat(torch, graph.replay, 0.05)
+    preheat(torch, graph.replay, 0.2)
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record()
     for _ in range(iters):
