@@ -55,14 +55,15 @@ constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 #ifndef PICO_DKDV_STAGES64
 #define PICO_DKDV_STAGES64 1
 #endif
-// Wave priority in the two middle stages of a dK/dV trip (those that mix MFMAs with softmax arithmetic): raised, so
-// that of the two waves of a SIMD the one with vector work to hide issues first (-1.5 % at head_dim 64)
+// Layout of the Q / dO tiles in LDS (elements of padding per row, elements of skew after every 4 rows): see KvCfg
 #ifndef PICO_DKDV_LDQPAD
 #define PICO_DKDV_LDQPAD 32
 #endif
 #ifndef PICO_DKDV_SKEW
 #define PICO_DKDV_SKEW 8
 #endif
+// Wave priority in the two middle stages of a dK/dV trip (those that mix MFMAs with softmax arithmetic): raised, so
+// that of the two waves of a SIMD the one with vector work to hide issues first (-1.5 % at head_dim 64)
 #ifndef PICO_DKDV_PRIO
 #define PICO_DKDV_PRIO 1
 #endif
@@ -96,7 +97,7 @@ struct KvCfg {
 template <int D>
 __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int ktile) {
   using C = KvCfg<D>;
-  constexpr int BM = C::BM, BN = C::BN, LDQ = C::LDQ;
+  constexpr int BM = C::BM, BN = C::BN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   auto tile_row = [](int r) { return r * C::LDQ + C::kSkew * (r >> 2); };   // element offset of a tile row
 
