@@ -647,6 +647,9 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
       const __bf16* sKs = sK + sub * BN * LDK;
       const __bf16* sVs = sV + sub * BN * LDK;
       f32x16 s_acc[BN / 32], dp_acc[BN / 32];
+      // the compiler's scheduler is asked for its MFMA / LDS-read interleaving of this block (-1 to -5 %; the key-split
+      // variant is better off without)
+      if constexpr (KS == 1) __builtin_amdgcn_iglp_opt(0);
 #pragma unroll
       for (int mb = 0; mb < BN / 32; ++mb) {
 #pragma unroll

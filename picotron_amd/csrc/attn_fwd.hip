@@ -229,6 +229,9 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
         if (a.causal && k0 > blk_q_lo + 31) continue;                  // whole 32x64 block is in the future
         // ---- S^T[key][query] for 64 keys x 32 queries
         f32x16 s_acc[BN / 32];
+        // Where no order is pinned by hand (head_dim 64), the compiler's scheduler is asked for its MFMA / LDS-read
+        // interleaving of this block (-1 % with 8 waves, -5 % with 4; the key-split variant is better off without)
+        if constexpr (C::kKDepth == 0 && KS == 1) __builtin_amdgcn_iglp_opt(0);
         // D = 128: the K fragments are fetched from LDS a fixed number of MFMAs ahead of their use.  An LDS read
         // takes several MFMA times to come back, so a read issued right before its MFMA leaves the matrix pipe
         // waiting for it (measured: +5 %).  At D = 64 the softmax arithmetic, not this wait, paces the loop, and the
