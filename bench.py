@@ -290,7 +290,7 @@ def bandwidth_extras(torch, ops, iters=50):
     return res
 
 
-def train_step_extra(torch, which="smollm_1p7b", steps=8, warmup=3, adamw="fp32_moments"):
+def train_step_extra(torch, which="smollm_1p7b", steps=10, warmup=3, adamw="fp32_moments"):
     """configs[2]: SmolLM-1.7B-shaped training step (24 layers, h 2048, 32 heads of 64, I 8192, V 49152), mbs 4, seq 1024;
     configs[3]: Llama-2-7B-shaped step (32 layers, h 4096, 32 heads of 128, I 11008, V 32000), mbs 1, seq 4096.
     bf16 parameters, random init, synthetic tokens.  adamw selects the optimizer's memory layout:
@@ -594,7 +594,7 @@ def main():
             extras["smollm_1p7b_train_step"] = train_step_extra(torch, "smollm_1p7b")
             extras["smollm_1p7b_train_step_fp32_master"] = train_step_extra(torch, "smollm_1p7b", adamw="fp32_master")
             extras["smollm_1p7b_train_step_reference_adamw_layout"] = train_step_extra(torch, "smollm_1p7b", adamw="reference")
-            extras["llama2_7b_train_step"] = train_step_extra(torch, "llama2_7b", steps=4, warmup=2)
+            extras["llama2_7b_train_step"] = train_step_extra(torch, "llama2_7b")
 
     line = {
         "metric": "causal ring-attn fwd+bwd TFLOP/s", "value": round(value, 2), "unit": "TFLOP/s",
