@@ -82,3 +82,65 @@ def test_seeded_shape_sweep(device):
         if bad:
             failures.append((case, B, Hq, Hkv, Sq, Sk, D, causal, q_offset, bad))
     assert not failures, failures
+
+
+def test_seeded_sweep_of_the_bandwidth_kernels(device):
+    """RMSNorm (both rounding orders, with and without the fused residual), SwiGLU and cross-entropy, forward and
+    backward, at 40 seeded sizes against torch in fp32 on the GPU."""
+    import torch.nn.functional as F
+    from picotron_amd import ops
+    rng = random.Random(7)
+    failures = []
+    for case in range(40):
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float32])
+        tol = 4e-2 if dtype == torch.bfloat16 else 2e-5
+        rows = rng.choice([1, 3, 17, 64, 255, 1000, 4096])
+        hidden = 8 * rng.choice([1, 9, 72, 96, 128, 256, 333, 512, 1024])
+        g = torch.Generator().manual_seed(1000 + case)
+        x = torch.randn(rows, hidden, generator=g).to(dtype).to(device)
+        res = torch.randn(rows, hidden, generator=g).to(dtype).to(device)
+        w = (torch.rand(hidden, generator=g) + 0.5).to(dtype).to(device)
+        dy = torch.randn(rows, hidden, generator=g).to(dtype).to(device)
+        eps = 1e-5
+        bad = []
+        # RMSNorm
+        for cts in (False, True):
+            y, rstd, _ = ops.rmsnorm_fwd(x, w, eps, cts)
+            xf = x.float().requires_grad_()
+            wf = w.float().requires_grad_()
+            normed = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+            want = (normed.to(dtype).float() * wf) if cts else normed * wf
+            if (y.float() - want).abs().max().item() > tol * max(1.0, want.abs().max().item()):
+                bad.append(f"rmsnorm_fwd cts={cts}")
+        y, rstd, h = ops.rmsnorm_fwd(x, w, eps, False, residual=res, want_residual_out=True)
+        hf = (x.float() + res.float()).to(dtype).float().requires_grad_()
+        wf = w.float().requires_grad_()
+        want = hf * torch.rsqrt(hf.pow(2).mean(-1, keepdim=True) + eps) * wf
+        gx, gw = torch.autograd.grad(want, (hf, wf), dy.float())
+        dx, dw = ops.rmsnorm_bwd(dy, h, w, rstd, dresidual=res)
+        if (h.float() - hf).abs().max().item() > 0 or rel_l2(y.float(), want.detach()) > 1e-2:
+            bad.append("rmsnorm_fwd residual")
+        if rel_l2(dx.float(), gx + res.float()) > 1e-2 or rel_l2(dw.float(), gw) > 1e-2:
+            bad.append("rmsnorm_bwd")
+        # SwiGLU
+        gf, uf = x.float().requires_grad_(), res.float().requires_grad_()
+        want = F.silu(gf) * uf
+        ggate, gup = torch.autograd.grad(want, (gf, uf), dy.float())
+        dgate, dup = ops.swiglu_bwd(dy, x, res)
+        if rel_l2(ops.swiglu_fwd(x, res).float(), want.detach()) > 1e-2 or rel_l2(dgate.float(), ggate) > 1e-2 or rel_l2(dup.float(), gup) > 1e-2:
+            bad.append("swiglu")
+        # cross-entropy over `hidden` classes
+        tgt = torch.randint(0, hidden, (rows,), generator=g).to(device)
+        if rows > 2:
+            tgt[1] = -100
+        lf = x.float().requires_grad_()
+        want_loss = F.cross_entropy(lf, tgt, ignore_index=-100, reduction="none")
+        loss_rows, lse = ops.cross_entropy_fwd(x, tgt)
+        count = max(int((tgt != -100).sum().item()), 1)
+        (gl,) = torch.autograd.grad(want_loss.sum() / count, lf)
+        dl = ops.cross_entropy_bwd(x, tgt, lse, torch.full((1,), 1.0 / count, device=device))
+        if (loss_rows - want_loss.detach()).abs().max().item() > 1e-3 or rel_l2(dl.float(), gl) > 1e-2:
+            bad.append("cross_entropy")
+        if bad:
+            failures.append((case, str(dtype), rows, hidden, bad))
+    assert not failures, failures
