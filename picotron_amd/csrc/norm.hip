@@ -333,10 +333,15 @@ void launch_dw_reduce(const float* partial, void* dweight, int dweight_dtype, in
     hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<float>, grid, block, 0, s, partial, static_cast<float*>(dweight), nparts, hidden);
 }
 
-int bwd_blocks(int64_t rows, int gpb) {
+// Blocks of the backward: as many as the rows need, up to a cap that shrinks with the row length -- every block ends by
+// writing (and the reduce kernel by reading) one row of the workspace, and at hidden 4096 the 512 blocks that are right
+// for hidden 2048 cost 19 % (measured at 4096 rows: 48.7 us with 512 blocks, 39.3 us with 256).
+int bwd_blocks(int64_t rows, int gpb, int hidden) {
   int64_t need = (rows + gpb - 1) / gpb;
   if (need < 1) need = 1;
-  return static_cast<int>(need < kMaxBwdBlocks ? need : kMaxBwdBlocks);
+  int cap = (1 << 20) / (hidden > 0 ? hidden : 1);
+  cap = cap < 64 ? 64 : (cap > kMaxBwdBlocks ? kMaxBwdBlocks : cap);
+  return static_cast<int>(need < cap ? need : cap);
 }
 
 // smallest supported NV >= need, or 0
@@ -396,14 +401,14 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
   const int nv_wave = pick_nv((nvec + 63) / 64, 8);
 #define PICO_BWD(G, NV)                                                            \
   {                                                                                \
-    const int blocks = bwd_blocks(rows, kBwdThreads / G);                          \
+    const int blocks = bwd_blocks(rows, kBwdThreads / G, hidden);                          \
     *blocks_out = blocks;                                                          \
     launch_bwd<T, G, NV>(dy, x, w, rstd, dres, dx, partial, blocks, rows, hidden, s); \
     return PICO_OK;                                                                \
   }
 #define PICO_BWD_WAVE(NV)                                                                              \
   {                                                                                                    \
-    const int blocks = bwd_blocks(rows, kBwdWaveThreads / kWave);                                      \
+    const int blocks = bwd_blocks(rows, kBwdWaveThreads / kWave, hidden);                                      \
     *blocks_out = blocks;                                                                              \
     const size_t lds = static_cast<size_t>(kBwdWaveThreads / kWave - 1) * hidden * sizeof(float);      \
     if (dres)                                                                                          \
