@@ -196,7 +196,9 @@ int pico_convert_f32(const float* src, void* dst, int64_t B, int64_t H, int64_t 
 /* ------------------------------------------------------------------ loss
  * replaces: F.cross_entropy(outputs.view(S*B, V), target_ids, reduction='mean')  train.py:46-49  and its autograd.
  * logits: [rows, vocab] with row pitch ld (elements; a multiple of 8 for bf16, 4 for fp32), dtype `dtype`;
- * targets: [rows] int64, each in [0, vocab) or equal to ignore_index (torch's default is -100).
+ * targets: [rows] int64, each in [0, vocab) or equal to ignore_index (torch's default is -100).  A target outside
+ *          [0, vocab) that is not ignore_index is never used as an index: the row is treated as ignored (loss 0,
+ *          gradient row 0) in both directions, where torch asserts on the device.
  * forward : loss[r] = logsumexp(logits[r]) - logits[r][target[r]] (0 for an ignored row) and lse[r], both fp32 [rows].
  *           The mean over the rows that are not ignored is left to the caller (one small reduction).
  * backward: dlogits[r][j] = (exp(logits[r][j] - lse[r]) - (j == target[r])) * scale[0], 0 for an ignored row;

@@ -2,11 +2,17 @@
 
 Same class name, methods, attributes and error behaviour (``Commit called twice`` :39, ``Wait called
 before commit`` :44), but the peer is the in-process ``LocalRing`` mailbox instead of
-``dist.batch_isend_irecv`` -- there is one GPU and no collective.  The communicator is told by its
-``msg`` which protocol it carries, exactly the three the reference opens (``context_parallel.py:21,60,61``):
+``dist.batch_isend_irecv`` -- there is one GPU and no collective.
 
-* ``"comm"`` / ``"kv_comm"``: K then V per ring step; step s delivers the chunk of rank (r-s-1) mod W.
-* ``"d_kv_comm"``: dK then dV per ring step; delivers the travelling fp32 accumulators.
+What a communicator carries is the K / V ring of ``context_parallel.py:21,60``: every ``send_recv`` of a ring
+step posts one tensor (K first, then V); ``wait`` completes the step by copying the peer's chunk into the
+receive buffers, which is the hop.  At ring step s rank r receives the chunk published by rank
+(r - s - 1) mod W.  ``msg`` is a label for the log lines, as in the reference.
+
+The reference's third ring (``d_kv_comm``, :61) moves the fp32 dK / dV accumulators from rank to rank.  Virtual
+ranks share one address space, so the accumulators do not travel: they live with the published chunk
+(``process_group_manager.GradBox``), every rank's backward adds its block there inside the kernel, and the chunk's
+autograd node returns the total after the last rank has added its part.
 """
 from __future__ import annotations
 
@@ -21,7 +27,10 @@ STEP, VERBOSE = 0, os.environ.get("VERBOSE", "0") == "1"
 
 
 class ContextCommunicate:
-    def __init__(self, msg: str = "", rank: Optional[int] = None, slot: Optional[int] = None):
+    def __init__(self, msg: str = "", rank: Optional[int] = None, slot: Optional[int] = None, chunks=None):
+        """`rank` / `slot` default to the rank being played and must be bound before the first wait(); `chunks`
+        ({rank: RingChunk}) serves the hops from chunks the caller already holds instead of the mailbox (a backward
+        pass reads the chunks its forward saw, whatever has been published since)."""
         mgr = pgm.process_group_manager
         self.msg = msg
         self.world_size = mgr.cp_world_size
@@ -30,19 +39,16 @@ class ContextCommunicate:
         self.recv_rank = (self.rank - 1) % self.world_size
         self._ring = mgr.cp_ring
         self._slot = slot
-        self._step = 0               # ring steps committed so far
+        self._chunks = chunks
+        self._step = 0               # ring steps completed so far
         self._pending: List[tuple] = []   # (sent tensor, receive buffer) of the open step
         self._active = None
         if VERBOSE:
             print(f"RingComm ({msg}) | initialized | RANK:{self.rank} | WORLD_SIZE:{self.world_size} | "
                   f"SEND_RANK:{self.send_rank} | RECV_RANK:{self.recv_rank}", flush=True)
 
-    # -- protocol helpers -------------------------------------------------------------
     def bind_slot(self, slot: int) -> None:
         self._slot = slot
-
-    def _is_grad_channel(self) -> bool:
-        return self.msg == "d_kv_comm"
 
     def send_recv(self, tensor_to_send, recv_tensor=None):
         result = torch.zeros_like(tensor_to_send) if recv_tensor is None else recv_tensor
@@ -56,37 +62,29 @@ class ContextCommunicate:
         if VERBOSE:
             print(f"RingComm | commit | STEP:{STEP} | RANK:{self.rank} | NUM_OPS:{len(self._pending)}", flush=True)
 
-    def wait(self):
+    def wait(self, needed: bool = True):
+        """Completes the open ring step.  `needed=False` says the arriving chunk will not be read (a causal ring
+        receives chunks of later ranks that it never uses): a chunk that is not in the mailbox is then skipped and
+        the receive buffers are filled with NaN, where `needed=True` raises."""
         if self._active is None:
             raise RuntimeError("Wait called before commit")
         W, r, s = self.world_size, self.rank, self._step
-        if self._slot is None:
+        if self._slot is None and self._chunks is None:
             raise RuntimeError("ContextCommunicate: no ring slot bound (use ring_attention / RingAttentionFunc)")
-        if self._is_grad_channel():
-            # what leaves is the accumulator of chunk (r - s) mod W; what arrives is that of chunk (r - s - 1) mod W
-            out_chunk, in_chunk = (r - s) % W, (r - s - 1) % W
-            sent = [t for t, _ in self._active]
-            key = (self._slot, out_chunk)
-            if s == 0 and key in self._ring.acc:
-                # a fresh accumulator meets contributions already left by ranks replayed earlier
-                for have, new in zip(self._ring.acc[key], sent):
-                    have.add_(new)
-            else:
-                self._ring.acc[key] = [t if t.dtype == torch.float32 else t.float() for t in sent]
-            self._ring.deposited.setdefault(key, set()).add(r)
-            have = self._ring.acc.get((self._slot, in_chunk))
-            for i, (_, buf) in enumerate(self._active):
-                if have is not None:
-                    buf.copy_(have[i])      # the hop: running total of the chunk arrives in the receive buffer
-                else:
-                    buf.zero_()
+        if len(self._active) > 2:
+            raise RuntimeError("ContextCommunicate: a ring step carries K and V (at most two tensors)")
+        src_rank = (r - s - 1) % W
+        held = self._chunks.get(src_rank) if self._chunks is not None else self._ring.chunks.get((self._slot, src_rank))
+        if held is None or held.k is None:
+            if needed:
+                if self._chunks is not None:
+                    raise RuntimeError(f"local cp ring: rank {r} was not given the K/V chunk of rank {src_rank}")
+                self._ring.fetch(self._slot, src_rank, r)      # raises, naming the chunk
+            for _, buf in self._active:
+                buf.fill_(float("nan"))
         else:
-            in_chunk = (r - s - 1) % W
-            have = self._ring.kv.get((self._slot, in_chunk))
-            if have is not None:
-                for (_, buf), src in zip(self._active, have):
-                    buf.copy_(src)          # the hop: the peer's chunk arrives in the receive buffer
-            # else: chunk of a rank that has not been replayed yet; under a causal mask it is never used
+            for (_, buf), src in zip(self._active, (held.k, held.v)):
+                buf.copy_(src.detach())                        # the hop: the peer's chunk arrives in the receive buffer
         self._step += 1
         self._active = None
         self._pending = []

@@ -780,22 +780,12 @@ __global__ __launch_bounds__(256) void attn_bwd_preprocess_kernel(const __bf16* 
   if (row < rows && v == 0) delta[row] = part;
 }
 
-template <typename K>
-int set_lds(K kernel, size_t bytes, const char* what) {
-  if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                          static_cast<int>(bytes)) != hipSuccess)
-    return fail(PICO_ERR_LAUNCH, "%s: cannot reserve %zu bytes of LDS", what, bytes);
-  return PICO_OK;
-}
-
 template <int D>
 int launch_dkdv(const BwdParams& p, hipStream_t s) {
   using C = KvCfg<D>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (int rc = set_lds(KvKernel<D>::fn, C::kLdsBytes, "pico_attn_bwd(dk/dv)")) return rc;
-    attr_set = true;
-  }
+  static std::atomic<bool> lds_reserved{false};
+  if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(KvKernel<D>::fn), C::kLdsBytes))
+    return fail(PICO_ERR_LAUNCH, "pico_attn_bwd(dk/dv): cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_ktiles = (p.a.Sk + C::BN - 1) / C::BN;
   // pairs only when they still fill the GPU (two workgroups per CU for D = 64, one for D = 128)
   BwdParams q = p;
@@ -809,11 +799,9 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
 template <int D, int NW, int KT, bool kDelta, int KS>
 int launch_dq_impl(const BwdParams& p, hipStream_t s) {
   using C = DqCfg<D, NW, KT, KS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (int rc = set_lds(&attn_bwd_dq_kernel<D, NW, KT, kDelta, KS>, C::kLdsBytes, "pico_attn_bwd(dq)")) return rc;
-    attr_set = true;
-  }
+  static std::atomic<bool> lds_reserved{false};
+  if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D, NW, KT, kDelta, KS>), C::kLdsBytes))
+    return fail(PICO_ERR_LAUNCH, "pico_attn_bwd(dq): cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
   hipLaunchKernelGGL((attn_bwd_dq_kernel<D, NW, KT, kDelta, KS>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, p);
   return PICO_OK;

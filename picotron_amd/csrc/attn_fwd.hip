@@ -407,13 +407,9 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
 template <int D, int QB, int NW, int KT, int KS = 1>
 int launch(const FwdParams& p, hipStream_t s) {
   using C = FwdCfg<D, QB, NW, KT, KS>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_fwd_kernel<D, QB, NW, KT, KS>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(C::kLdsBytes)) != hipSuccess)
-      return fail(PICO_ERR_LAUNCH, "pico_attn_fwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
-    attr_set = true;
-  }
+  static std::atomic<bool> lds_reserved{false};
+  if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(&attn_fwd_kernel<D, QB, NW, KT, KS>), C::kLdsBytes))
+    return fail(PICO_ERR_LAUNCH, "pico_attn_fwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
   FwdParams q = p;
   q.pair_order = p.a.causal && n_qtiles >= 2 && static_cast<int64_t>(p.a.Hq) * p.a.B * n_qtiles <= 512;

@@ -2,6 +2,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <atomic>
 #include "../../include/picotron_amd.h"
 
 namespace pico {
@@ -86,5 +87,16 @@ template <> struct io<float> {
 };
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Raises a kernel's dynamic-LDS limit the first time the kernel is launched.  Host threads may race here (autograd
+// runs backward on a thread of its own): the flag is atomic and the HIP call is idempotent, so two first callers
+// both make it and both proceed only after it has succeeded.
+inline bool reserve_lds_once(std::atomic<bool>& done, const void* kernel, size_t bytes) {
+  if (done.load(std::memory_order_acquire)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) != hipSuccess)
+    return false;
+  done.store(true, std::memory_order_release);
+  return true;
+}
 
 }  // namespace pico

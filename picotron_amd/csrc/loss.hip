@@ -1,7 +1,8 @@
 // Cross-entropy over the vocabulary: one workgroup per token row.
 //   forward : lse = logsumexp(row), loss = lse - row[target]      (one read of the logits)
 //   backward: dlogits = (exp(row - lse) - onehot(target)) * scale  (one read, one write)
-// fp32 arithmetic on bf16 or fp32 logits; rows whose target equals ignore_index contribute nothing.
+// fp32 arithmetic on bf16 or fp32 logits; rows whose target equals ignore_index -- or lies outside [0, vocab), which
+// no load may follow -- contribute nothing: loss 0, gradient row 0.
 #include "common.h"
 
 namespace pico {
@@ -59,7 +60,8 @@ __global__ __launch_bounds__(kThreads) void ce_fwd_kernel(const T* __restrict__ 
     const float lse = (bm + fast_log2(bs)) * kLn2;
     const int64_t t = targets[row];
     lse_out[row] = lse;
-    loss[row] = (t == ignore_index) ? 0.f : lse - static_cast<float>(x[t]);
+    const bool counts = t != ignore_index && t >= 0 && t < vocab;
+    loss[row] = counts ? lse - static_cast<float>(x[t]) : 0.f;
   }
 }
 
@@ -73,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void ce_bwd_kernel(const T* __restrict__ 
   const T* x = logits + row * ld;
   T* d = dlogits + row * dld;
   const int64_t t = targets[row];
-  const float scale = (t == ignore_index) ? 0.f : *scale_ptr;
+  const float scale = (t != ignore_index && t >= 0 && t < vocab) ? *scale_ptr : 0.f;
   const float l2 = lse[row] * kLog2e;
   const int nvec = vocab / V;
   for (int v = threadIdx.x; v < nvec; v += kThreads) {

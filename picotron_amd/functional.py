@@ -29,11 +29,15 @@ class RMSNormResidualFunc(torch.autograd.Function):
     def forward(ctx, x, residual, weight, eps):
         y, rstd, h = ops.rmsnorm_fwd(x, weight, eps, False, residual=residual, want_residual_out=True)
         ctx.save_for_backward(h, weight, rstd)
+        ctx.set_materialize_grads(False)    # the last norm's h has no consumer: no zero tensor is made for it
         return y, h
 
     @staticmethod
     def backward(ctx, dy, dh):
         h, weight, rstd = ctx.saved_tensors
+        if dy is None:
+            # only the residual stream carried a gradient: it passes through the add unchanged
+            return dh, dh, None, None
         # dh, the gradient that reached h without passing the norm, is added inside the kernel
         dx, dw = ops.rmsnorm_bwd(dy, h, weight, rstd, dresidual=dh, dw_dtype=weight.dtype)
         return dx, dx, dw, None
@@ -96,7 +100,8 @@ class CrossEntropyFunc(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logits, targets, ignore_index=-100):
         loss_rows, lse = ops.cross_entropy_fwd(logits, targets, ignore_index)
-        count = (targets != ignore_index).sum().clamp(min=1).to(torch.float32)
+        # rows that count: not ignored and a valid index (the kernels skip a target outside [0, vocab) as well)
+        count = ((targets != ignore_index) & (targets >= 0) & (targets < logits.size(-1))).sum().clamp(min=1).to(torch.float32)
         ctx.save_for_backward(logits, targets, lse, count)
         ctx.ignore_index = ignore_index
         return loss_rows.sum() / count

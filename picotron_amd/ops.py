@@ -357,15 +357,20 @@ def attn_bwd(dout, q, k, v, lse, delta, sm_scale: float, causal: bool, q_offset:
     return dq, dk, dv
 
 
-def convert_f32(src: torch.Tensor, dtype, like: Optional[torch.Tensor] = None, bshd: bool = False) -> torch.Tensor:
-    """fp32 contiguous [B,H,S,D] -> dtype; laid out like `like` (same strides), as a view over [B,S,H,D]
-    memory (bshd=True), or contiguous."""
+def convert_f32(src: torch.Tensor, dtype, like: Optional[torch.Tensor] = None, bshd: bool = False,
+                strides=None) -> torch.Tensor:
+    """fp32 contiguous [B,H,S,D] -> dtype; laid out like `like` (same strides) or with the given `strides` (of a
+    dense layout with a unit D stride), as a view over [B,S,H,D] memory (bshd=True), or contiguous."""
     _dev(src, like)
     if src.dtype != torch.float32 or not src.is_contiguous() or src.dim() != 4:
         raise RuntimeError("convert_f32: src must be a contiguous fp32 [B,H,S,D] tensor")
     B, H, S, D = src.shape
     if bshd:
         dst = empty_bshd(B, H, S, D, dtype, src.device)
+    elif strides is not None:
+        dst = torch.empty_strided(src.shape, tuple(strides), dtype=dtype, device=src.device)
+        if dst.stride(-1) != 1 or not _dense(dst):
+            raise RuntimeError("convert_f32: strides must describe a dense layout with a unit D stride")
     elif like is not None and _dense(like) and like.stride(-1) == 1:
         dst = torch.empty_strided(src.shape, like.stride(), dtype=dtype, device=src.device)
     else:

@@ -14,31 +14,62 @@ from typing import Dict, Optional, Tuple
 import torch
 
 
+class GradBox:
+    """fp32 dK / dV accumulators of one published chunk: what travels round the ring in the reference
+    (``context_parallel.py:85-106``).  Every rank's backward adds its block here; the chunk's own autograd node
+    hands the total back once all of them have run."""
+
+    __slots__ = ("dk", "dv")
+
+    def __init__(self):
+        self.dk: Optional[torch.Tensor] = None
+        self.dv: Optional[torch.Tensor] = None
+
+
+class RingChunk:
+    """The K / V chunk one virtual rank holds at ring step 0 of one ring_attention call."""
+
+    __slots__ = ("slot", "rank", "src_k", "src_v", "k", "v", "grads")
+
+    def __init__(self, slot: int, rank: int, src_k: torch.Tensor, src_v: torch.Tensor):
+        self.slot, self.rank = slot, rank
+        self.src_k, self.src_v = src_k, src_v      # what the caller passed (to recognise a chunk staged ahead)
+        self.k, self.v = src_k, src_v              # what peers read; replaced by autograd-tracked aliases on publish
+        self.grads = GradBox()
+
+
+def _same_tensor(a: torch.Tensor, b: torch.Tensor) -> bool:
+    return a is b or (a.data_ptr() == b.data_ptr() and a.shape == b.shape and a.stride() == b.stride()
+                      and a.dtype == b.dtype and a._version == b._version)
+
+
 class LocalRing:
     """Mailbox that stands in for the cp ring's P2P hops (``cp_communications.py:22-41``).
 
-    K/V: the chunk a rank holds at ring step 0 is published under (slot, rank); what rank r
-    receives at step s is the chunk published by rank (r - s - 1) mod W for the same slot
-    (every hop moves a chunk one rank up, ``process_group_manager.py:43-44``).  A slot is one call
-    site of ring_attention within a rank's pass (layer i of the model), numbered by call order.
+    The chunk a rank holds at ring step 0 is published under (slot, rank); what rank r receives at step s is
+    the chunk published by rank (r - s - 1) mod W for the same slot (every hop moves a chunk one rank up,
+    ``process_group_manager.py:43-44``).  A slot is one call site of ring_attention within a rank's pass
+    (layer i of the model), numbered by call order.
 
-    dK/dV: ``acc[(slot, c)]`` is the travelling fp32 accumulator of chunk c.  A rank receives the
-    running total and sends back total + its own block, so replaying ranks one after another leaves
-    the same sums the real ring produces (``context_parallel.py:85-106``).
+    A pass is one play of the ranks.  Publishing a (slot, rank) that the mailbox already holds means a new pass
+    has begun (the next micro-batch or optimiser step): everything from the old pass is dropped first, so a
+    chunk of an earlier pass can never be delivered.  Asking for a chunk that is not there raises.
+
+    Under a causal mask rank r reads chunks 0..r, so playing the ranks in ascending order needs nothing else.
+    Without a mask every rank reads every chunk; ``stage_kv`` lets the caller hand over all ranks' K / V
+    before the first rank is played.
     """
 
     def __init__(self, world_size: int):
         self.world_size = world_size
-        self.kv: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
-        self.acc: Dict[Tuple[int, int], list] = {}
-        self.deposited: Dict[Tuple[int, int], set] = {}
+        self.chunks: Dict[Tuple[int, int], RingChunk] = {}
         self._next_slot = 0
 
     def reset(self) -> None:
-        """Forget every published chunk and accumulator (call between optimiser steps)."""
-        self.kv.clear()
-        self.acc.clear()
-        self.deposited.clear()
+        """Forget every published chunk.  The mailbox keeps the last pass's K / V alive until the next pass begins
+        (a later rank, or a rank's forward that follows another rank's backward, may still read them); call this to
+        free them earlier."""
+        self.chunks.clear()
         self._next_slot = 0
 
     def begin_rank(self) -> None:
@@ -50,8 +81,31 @@ class LocalRing:
         self._next_slot += 1
         return s
 
-    def publish_kv(self, slot: int, rank: int, k: torch.Tensor, v: torch.Tensor) -> None:
-        self.kv[(slot, rank)] = (k, v)
+    def publish_kv(self, slot: int, rank: int, k: torch.Tensor, v: torch.Tensor) -> RingChunk:
+        key = (slot, rank)
+        held = self.chunks.get(key)
+        if held is not None:
+            if _same_tensor(held.src_k, k) and _same_tensor(held.src_v, v):
+                return held                      # staged ahead of the play by stage_kv
+            self.chunks.clear()                  # a new pass: nothing of the old one may be delivered
+        chunk = RingChunk(slot, rank, k, v)
+        self.chunks[key] = chunk
+        return chunk
+
+    def stage_kv(self, rank: int, k: torch.Tensor, v: torch.Tensor, slot: int = 0) -> RingChunk:
+        """Hand over rank `rank`'s chunk before that rank is played (needed when attention is not causal: every
+        rank reads every chunk).  ring_attention recognises the same tensors when the rank's turn comes."""
+        from picotron_amd.context_parallel.context_parallel import publish_chunk
+        return publish_chunk(self, slot, rank, k, v)
+
+    def fetch(self, slot: int, rank: int, reader: int) -> RingChunk:
+        chunk = self.chunks.get((slot, rank))
+        if chunk is None or chunk.k is None:
+            raise RuntimeError(
+                f"local cp ring: rank {reader} needs the K/V chunk of rank {rank} (ring_attention call {slot} of the "
+                f"pass), which has not been published in this pass; play the ranks in ascending order (causal) or "
+                f"hand all chunks over first with cp_ring.stage_kv(rank, k, v)")
+        return chunk
 
 
 class ProcessGroupManager:

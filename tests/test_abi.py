@@ -109,33 +109,6 @@ def test_process_group_manager_stand_in():
     pgm.setup_process_group_manager(1, 1, 1, 1)
 
 
-def test_local_ring_kv_and_grad_mailbox_on_cpu():
-    """The mailbox protocol itself is host logic: replay two virtual ranks with CPU tensors."""
-    import picotron_amd.process_group_manager as pgm
-    from picotron_amd.context_parallel.cp_communications import ContextCommunicate
-    mgr = pgm.setup_process_group_manager(1, 2, 1, 1)
-    k0, k1 = torch.full((2,), 10.0), torch.full((2,), 11.0)
-    mgr.cp_ring.publish_kv(0, 0, k0, k0)
-    mgr.cp_ring.publish_kv(0, 1, k1, k1)
-    c = ContextCommunicate("comm", rank=1, slot=0)
-    got = c.send_recv(k1)
-    c.commit()
-    c.wait()
-    assert torch.equal(got, k0)                                    # rank 1 receives rank 0's chunk at step 0
-    # gradients: rank 1 first (descending), then rank 0; chunk 0's accumulator must end as the sum
-    g1 = ContextCommunicate("d_kv_comm", rank=1, slot=0)
-    a = g1.send_recv(torch.full((2,), 1.0)); g1.commit(); g1.wait()            # step 0: sends chunk 1, receives chunk 0 (empty)
-    assert torch.equal(a, torch.zeros(2))
-    b = g1.send_recv(a + 5.0); g1.commit(); g1.wait()                          # step 1: sends chunk 0 (+5), receives chunk 1
-    assert torch.equal(b, torch.full((2,), 1.0))
-    g0 = ContextCommunicate("d_kv_comm", rank=0, slot=0)
-    a = g0.send_recv(torch.full((2,), 7.0)); g0.commit(); g0.wait()            # step 0: fresh chunk 0 meets rank 1's 5
-    b = g0.send_recv(a); g0.commit(); g0.wait()                                # step 1: pass-through of chunk 1; receives chunk 0
-    assert torch.equal(b, torch.full((2,), 12.0))
-    assert mgr.cp_ring.deposited[(0, 0)] == {0, 1}
-    pgm.setup_process_group_manager(1, 1, 1, 1)
-
-
 C_PROGRAM = r"""
 #include <stdio.h>
 #include <string.h>

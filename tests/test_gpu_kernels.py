@@ -626,6 +626,32 @@ def test_cross_entropy_against_oracle(ops, device, rows, vocab, dtype):
     assert xd.grad[1].abs().max().item() == 0.0
 
 
+def test_cross_entropy_target_out_of_range_is_skipped_not_read(ops, device):
+    """A target outside [0, vocab) that is not ignore_index (a pad id, a -100 with another ignore_index) must never be
+    used as an index: the row counts as ignored in both directions, and the mean is over the rows that count."""
+    from oracle import layers as OL
+    from picotron_amd.functional import cross_entropy
+    g = torch.Generator().manual_seed(4)
+    rows, vocab = 12, 515
+    x = (torch.randn(rows, vocab, generator=g) * 3).to(torch.bfloat16)
+    t = torch.randint(0, vocab, (rows,), generator=g)
+    bad = {0: -5, 3: vocab, 7: vocab + (1 << 40), 9: -100}
+    for r, val in bad.items():
+        t[r] = val
+    pitch = (vocab + 7) // 8 * 8
+    xd = torch.zeros(rows, pitch, dtype=torch.bfloat16, device=device)[:, :vocab].copy_(x.to(device)).requires_grad_()
+    loss = cross_entropy(xd, t.to(device), ignore_index=-1)      # -100 is NOT the ignore index here
+    loss.backward()
+    loss_rows, _ = ops.cross_entropy_fwd(xd.detach(), t.to(device), -1)
+    keep = torch.tensor([r not in bad for r in range(rows)])
+    want, _ = OL.cross_entropy(x[keep], t[keep])
+    assert abs(loss.item() - want.item()) <= 2e-5 * max(1.0, abs(want.item()))
+    for r in bad:
+        assert loss_rows[r].item() == 0.0 and xd.grad[r].abs().max().item() == 0.0
+    gw = OL.cross_entropy_backward(x[keep], t[keep], 1.0)
+    assert maxabs(xd.grad[keep.to(device)], gw) <= 2 ** -8 * gw.abs().max().item() + 1e-9
+
+
 def test_fused_adamw_overlapped_with_backward_gives_the_same_update(device):
     """overlap_with_backward updates each parameter from a hook on a second stream; same numbers as step()."""
     from picotron_amd.optim import FusedAdamW

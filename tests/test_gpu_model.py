@@ -93,17 +93,88 @@ def test_ring_attention_func_every_rank(pgm1, device):
     pgm.setup_process_group_manager(1, 1, 1, 1)
 
 
-def test_ring_backward_wrong_order_is_refused(pgm1, device):
+def _ring_case(device, W, causal, seed, B=2, H=4, Hkv=2, Sc=64, D=64):
+    g = torch.Generator().manual_seed(seed)
+    S = W * Sc
+    q, k, v, do = (torch.randn(B, h, S, D, generator=g).to(torch.bfloat16) for h in (H, Hkv, Hkv, H))
+    scale = 1 / math.sqrt(D)
+    rep = H // Hkv
+    w_o, w_l = OR.all_ranks_forward(q.float(), k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1),
+                                    W, scale, causal)
+    w_dq, w_dk, w_dv = OR.all_ranks_backward(do.float(), q.float(), k.float().repeat_interleave(rep, 1),
+                                             v.float().repeat_interleave(rep, 1), w_o, w_l, W, scale, causal)
+    fold = lambda t: t.view(B, Hkv, rep, S, D).sum(2)
+    return (q, k, v, do, scale), (w_o, w_dq, fold(w_dk), fold(w_dv))
+
+
+def _play_ring(mgr, cp, qd, kd, vd, scale, causal, W, order=None, stage=False):
+    Sc = qd.size(2) // W
+    ks = [kd[:, :, r * Sc:(r + 1) * Sc] for r in range(W)]
+    vs = [vd[:, :, r * Sc:(r + 1) * Sc] for r in range(W)]
+    if stage:
+        for r in range(W):
+            mgr.cp_ring.stage_kv(r, ks[r], vs[r])
+    outs = {}
+    for r in (order or range(W)):
+        mgr.set_cp_rank(r)
+        outs[r] = cp.ring_attention(qd[:, :, r * Sc:(r + 1) * Sc], ks[r], vs[r], scale, causal)
+    return [outs[r] for r in range(W)]
+
+
+def test_ring_two_passes_on_one_manager(pgm1, device):
+    """Two forward + backward passes on ONE manager (consecutive micro-batches): the second must be as right as the
+    first -- nothing of pass 1 may be left in the mailbox or in a dK / dV accumulator."""
     import picotron_amd.process_group_manager as pgm
     from picotron_amd.context_parallel import context_parallel as cp
-    mgr = pgm.setup_process_group_manager(1, 2, 1, 1)
-    x = [torch.randn(1, 1, 64, 64, device=device, dtype=torch.bfloat16, requires_grad=True) for _ in range(2)]
-    outs = []
-    for r in range(2):
-        mgr.set_cp_rank(r)
-        outs.append(cp.ring_attention(x[r], x[r], x[r], 0.125, True))
-    with pytest.raises(RuntimeError, match="have not added"):
-        outs[0].float().sum().backward()
+    W = 4
+    mgr = pgm.setup_process_group_manager(1, W, 1, 1)
+    for seed in (21, 22):
+        (q, k, v, do, scale), (w_o, w_dq, w_dk, w_dv) = _ring_case(device, W, True, seed)
+        qd, kd, vd = (t.to(device).requires_grad_() for t in (q, k, v))
+        out = torch.cat(_play_ring(mgr, cp, qd, kd, vd, scale, True, W), dim=2)
+        (out.float() * do.to(device).float()).sum().backward()
+        assert maxabs(out, w_o) <= 2e-2, seed
+        assert rel_l2(qd.grad, w_dq) <= 1e-2 and rel_l2(kd.grad, w_dk) <= 1e-2 and rel_l2(vd.grad, w_dv) <= 1e-2, seed
+    pgm.setup_process_group_manager(1, 1, 1, 1)
+
+
+@pytest.mark.parametrize("W", [2, 4])
+def test_ring_attention_func_without_mask(pgm1, device, W):
+    """is_causal=False with W > 1 (``context_parallel.py:36,78``): every rank runs every ring step; all chunks are
+    staged before the ranks are played; forward and backward against the CPU oracle's ring."""
+    import picotron_amd.process_group_manager as pgm
+    from picotron_amd.context_parallel import context_parallel as cp
+    mgr = pgm.setup_process_group_manager(1, W, 1, 1)
+    (q, k, v, do, scale), (w_o, w_dq, w_dk, w_dv) = _ring_case(device, W, False, 30 + W)
+    for order in (list(range(W)), list(reversed(range(W)))):
+        qd, kd, vd = (t.to(device).requires_grad_() for t in (q, k, v))
+        out = torch.cat(_play_ring(mgr, cp, qd, kd, vd, scale, False, W, order=order, stage=True), dim=2)
+        (out.float() * do.to(device).float()).sum().backward()
+        assert maxabs(out, w_o) <= 2e-2
+        assert rel_l2(qd.grad, w_dq) <= 1e-2 and rel_l2(kd.grad, w_dk) <= 1e-2 and rel_l2(vd.grad, w_dv) <= 1e-2
+    # nothing staged: refused, not computed from zeros
+    mgr.cp_ring.reset()
+    with pytest.raises(RuntimeError, match="has not been published"):
+        _play_ring(mgr, cp, qd, kd, vd, scale, False, W)
+    pgm.setup_process_group_manager(1, 1, 1, 1)
+
+
+def test_ring_backward_one_rank_at_a_time(pgm1, device):
+    """Each rank's loss differentiated by its own backward call, last rank first and first rank first."""
+    import picotron_amd.process_group_manager as pgm
+    from picotron_amd.context_parallel import context_parallel as cp
+    W = 4
+    mgr = pgm.setup_process_group_manager(1, W, 1, 1)
+    (q, k, v, do, scale), (w_o, w_dq, w_dk, w_dv) = _ring_case(device, W, True, 40, B=1)
+    Sc = q.size(2) // W
+    dod = do.to(device).float()
+    for order in ([3, 2, 1, 0], [0, 1, 2, 3]):
+        qd, kd, vd = (t.to(device).requires_grad_() for t in (q, k, v))
+        outs = _play_ring(mgr, cp, qd, kd, vd, scale, True, W)
+        for r in order:
+            (outs[r].float() * dod[:, :, r * Sc:(r + 1) * Sc]).sum().backward()
+        # four bf16 partial sums per leaf instead of one fp32 sum: a little looser than the one-call bound
+        assert rel_l2(qd.grad, w_dq) <= 1e-2 and rel_l2(kd.grad, w_dk) <= 1.5e-2 and rel_l2(vd.grad, w_dv) <= 1.5e-2, order
     pgm.setup_process_group_manager(1, 1, 1, 1)
 
 
@@ -132,6 +203,27 @@ def test_update_out_and_lse_api(pgm1, device):
         w_o, w_l = OR.merge(w_o, w_l, o.float(), l)
     assert out.dtype == torch.float32 and lse.shape == (1, 2, 9, 1)
     assert maxabs(out, w_o) <= 1e-5 and maxabs(lse, w_l) <= 1e-5
+
+
+def test_update_out_and_lse_slice_branch(pgm1, device):
+    """The slice_ form (``context_parallel.py:164-168, 182-183``): only the selected rows of the running (out, lse)
+    are merged with the block; the others keep their bits."""
+    from picotron_amd.context_parallel import context_parallel as cp
+    g = torch.Generator().manual_seed(8)
+    B, H, S, D = 2, 3, 24, 64
+    out0 = torch.randn(B, H, S, D, generator=g)
+    lse0 = torch.randn(B, H, S, 1, generator=g)
+    for slice_ in ((slice(None), slice(None), slice(8, 16)), (slice(0, 1), slice(1, 3), slice(None, None, 2))):
+        rows = out0[slice_].shape
+        bo = torch.randn(rows, generator=g).to(torch.bfloat16)
+        bl = torch.randn(rows[:-1], generator=g)
+        w_o, w_l = OR.merge(out0.clone(), lse0.clone(), bo.float(), bl, slice_=slice_)
+        out, lse = cp.update_out_and_lse(out0.to(device), lse0.to(device), bo.to(device), bl.to(device), slice_=slice_)
+        assert out.shape == out0.shape and lse.shape == lse0.shape
+        assert maxabs(out, w_o) <= 1e-5 and maxabs(lse, w_l) <= 1e-5
+        untouched = torch.ones(B, H, S, dtype=torch.bool)
+        untouched[slice_] = False
+        assert torch.equal(out.cpu()[untouched], out0[untouched]) and torch.equal(lse.cpu()[untouched], lse0[untouched])
 
 
 def test_update_rope_for_context_parallel_exact(device):
@@ -214,7 +306,6 @@ def test_model_cp4_virtual_ranks_equals_cp1(pgm1, device):
     assert abs(total.item() - loss1.item()) <= 2e-2
     for (n1, p1), (n4, p4) in zip(m1.named_parameters(), m4.named_parameters()):
         assert rel_l2(p4.grad, p1.grad) <= 5e-2, n1
-    mgr.cp_ring.reset()
     pgm.setup_process_group_manager(1, 1, 1, 1)
     os.environ["CONTEXT_PARALLEL"] = "0"
 
