@@ -77,6 +77,23 @@ int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const fl
                      void* dx, void* dweight, int dweight_dtype, void* workspace, int64_t workspace_bytes,
                      int64_t rows, int64_t hidden, int dtype, void* stream);
 
+/* pico_rmsnorm_bwd without the workspace argument: the one entry point that allocates nothing and needs nothing
+ * allocated for it.  It has no counterpart in the reference; it is for callers that cannot call hipMalloc or hand over
+ * scratch memory -- code under HIP graph capture, tight serving loops, harnesses that forbid allocation.  The
+ * per-block partial sums of dweight go to a static device array inside the library (4 MiB per GPU, held until the
+ * process ends) instead of the caller's workspace; arguments, kernels and results are otherwise those of
+ * pico_rmsnorm_bwd, bit for bit.  The device the pointers live on must be the current device.
+ * Limit: the launch's partial sums must fit the array -- pico_rmsnorm_bwd_static_max_bytes(); every hidden <= 16384
+ * the kernels accept does, whatever `rows` is -- otherwise PICO_ERR_WORKSPACE is returned and nothing is launched.
+ * All calls on one GPU share that array: calls that overlap in time on one GPU (two streams, two host threads)
+ * race on it and must be serialised by the caller.  Nothing in it needs clearing between calls: a launch writes
+ * every partial sum it later reads.
+ */
+int64_t pico_rmsnorm_bwd_static_max_bytes(void);
+int pico_rmsnorm_bwd_static(const void* dy, const void* x, const void* weight, const float* rstd,
+                            const void* dresidual, void* dx, void* dweight, int dweight_dtype,
+                            int64_t rows, int64_t hidden, int dtype, void* stream);
+
 /* ------------------------------------------------------------------ RoPE
  * replaces: apply_rotary_pos_emb  model.py:12-19  and the flash-attn rotary call model.py:136-137
  *           (non-interleaved: element i pairs with i + D/2), with the row selection of

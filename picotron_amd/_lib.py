@@ -32,6 +32,8 @@ SIGNATURES = {
     "pico_rmsnorm_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _I64, _I64, c_float, c_int, c_int, _P]),
     "pico_rmsnorm_bwd_workspace_bytes": (_I64, [_I64, _I64]),
     "pico_rmsnorm_bwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, _P, _I64, _I64, _I64, c_int, _P]),
+    "pico_rmsnorm_bwd_static_max_bytes": (_I64, []),
+    "pico_rmsnorm_bwd_static": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_int, _I64, _I64, c_int, _P]),
     "pico_rope": (c_int, [_P, _P, _P, _P] + [_I64] * 4 + [_I64] * 6 + [_I64, _I64, c_int, c_int, c_int, _P]),
     "pico_swiglu_fwd": (c_int, [_P, _P, _P] + [_I64] * 5 + [c_int, _P]),
     "pico_swiglu_bwd": (c_int, [_P] * 5 + [_I64] * 7 + [c_int, _P]),

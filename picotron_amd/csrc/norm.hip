@@ -3,6 +3,12 @@
 // stays in registers between the reduction and the normalisation so HBM is touched once.
 #include "common.h"
 
+// Scratch of pico_rmsnorm_bwd_static, the entry point that allocates nothing: the per-block partial sums of dweight
+// that pico_rmsnorm_bwd keeps in the caller's workspace.  4 MiB per GPU, held until the process ends.  In host code
+// this name is only a handle: the device address comes from hipGetSymbolAddress (static_scratch() below).
+constexpr size_t kStaticScratchFloats = size_t(1) << 20;
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
 namespace pico {
 namespace {
 
@@ -447,6 +453,19 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
   return fail(PICO_ERR_SHAPE, "pico_rmsnorm_bwd: hidden=%d too large", hidden);
 }
 
+// Bytes of partial sums one backward launch writes: (blocks it will use) x hidden floats -- the same choice of
+// kernel and grid as dispatch_bwd.
+int64_t bwd_partial_bytes(int64_t rows, int64_t hidden, int dtype) {
+  const int vec = dtype == PICO_BF16 ? 8 : 4;
+  const int nvec = static_cast<int>(hidden / vec);
+  const int nv_wave = pick_nv((nvec + 63) / 64, 8);
+  int gpb;
+  if (nv_wave && static_cast<size_t>(hidden) * 3 * sizeof(float) <= 65536) gpb = kBwdWaveThreads / kWave;
+  else if (nv_wave) gpb = kBwdThreads / 64;
+  else gpb = kBwdThreads / 256;
+  return static_cast<int64_t>(bwd_blocks(rows, gpb, static_cast<int>(hidden))) * hidden * static_cast<int64_t>(sizeof(float));
+}
+
 int check_common(const char* fn, int64_t rows, int64_t hidden, int dtype) {
   if (dtype != PICO_BF16 && dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: dtype code %d not supported", fn, dtype);
   const int vec = dtype == PICO_BF16 ? 8 : 4;
@@ -484,34 +503,88 @@ extern "C" int64_t pico_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t hidden
   return static_cast<int64_t>(kMaxBwdBlocks) * hidden * static_cast<int64_t>(sizeof(float));
 }
 
-extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
-                                const void* dresidual, void* dx, void* dweight, int dweight_dtype, void* workspace,
-                                int64_t workspace_bytes, int64_t rows, int64_t hidden, int dtype, void* stream) {
-  if (int rc = check_common("pico_rmsnorm_bwd", rows, hidden, dtype)) return rc;
+namespace {
+
+// Everything of the backward but the question of where the partial sums live.  `partial_bytes` is what the caller's
+// buffer holds; the launch needs bwd_partial_bytes(rows, hidden) of it.
+int rmsnorm_bwd_impl(const char* fn, const void* dy, const void* x, const void* weight, const float* rstd,
+                     const void* dresidual, void* dx, void* dweight, int dweight_dtype, float* partial,
+                     int64_t partial_bytes, int64_t rows, int64_t hidden, int dtype, hipStream_t s) {
+  if (int rc = check_common(fn, rows, hidden, dtype)) return rc;
   if (dweight_dtype != PICO_BF16 && dweight_dtype != PICO_F32)
-    return fail(PICO_ERR_DTYPE, "pico_rmsnorm_bwd: dweight dtype code %d not supported", dweight_dtype);
-  if (!dweight) return fail(PICO_ERR_NULL, "pico_rmsnorm_bwd: dweight is required");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+    return fail(PICO_ERR_DTYPE, "%s: dweight dtype code %d not supported", fn, dweight_dtype);
+  if (!dweight) return fail(PICO_ERR_NULL, "%s: dweight is required", fn);
   if (rows == 0) {  // empty sum: dweight = 0 (the reduce kernel with no partials writes zeros)
     launch_dw_reduce(nullptr, dweight, dweight_dtype, 0, static_cast<int>(hidden), s);
-    return check_launch("pico_rmsnorm_bwd(empty)");
+    return check_launch(fn);
   }
-  if (!dy || !x || !weight || !rstd || !dx || !workspace)
-    return fail(PICO_ERR_NULL, "pico_rmsnorm_bwd: dy, x, weight, rstd, dx and workspace are required");
-  if (workspace_bytes < pico_rmsnorm_bwd_workspace_bytes(rows, hidden))
-    return fail(PICO_ERR_WORKSPACE, "pico_rmsnorm_bwd: workspace has %lld bytes, needs %lld",
-                static_cast<long long>(workspace_bytes),
-                static_cast<long long>(pico_rmsnorm_bwd_workspace_bytes(rows, hidden)));
-  if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(workspace) ||
+  if (!dy || !x || !weight || !rstd || !dx || !partial)
+    return fail(PICO_ERR_NULL, "%s: dy, x, weight, rstd, dx and the partial-sum buffer are required", fn);
+  const int64_t need = bwd_partial_bytes(rows, hidden, dtype);
+  if (partial_bytes < need)
+    return fail(PICO_ERR_WORKSPACE, "%s: the partial-sum buffer has %lld bytes, rows=%lld hidden=%lld need %lld", fn,
+                static_cast<long long>(partial_bytes), static_cast<long long>(rows), static_cast<long long>(hidden),
+                static_cast<long long>(need));
+  if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(partial) ||
       !aligned16(dresidual))
-    return fail(PICO_ERR_ALIGN, "pico_rmsnorm_bwd: pointers must be 16-byte aligned");
+    return fail(PICO_ERR_ALIGN, "%s: pointers must be 16-byte aligned", fn);
   int blocks = 0;
-  float* partial = static_cast<float*>(workspace);
   int rc = dtype == PICO_BF16
                ? dispatch_bwd<__bf16>(dy, x, weight, rstd, dresidual, dx, partial, rows, static_cast<int>(hidden), s, &blocks)
                : dispatch_bwd<float>(dy, x, weight, rstd, dresidual, dx, partial, rows, static_cast<int>(hidden), s, &blocks);
   if (rc) return rc;
-  if (int lrc = check_launch("pico_rmsnorm_bwd")) return lrc;
+  if (int lrc = check_launch(fn)) return lrc;
   launch_dw_reduce(partial, dweight, dweight_dtype, blocks, static_cast<int>(hidden), s);
-  return check_launch("pico_rmsnorm_bwd(dweight reduce)");
+  return check_launch(fn);
+}
+
+// Device address of `scratch` on the current GPU, looked up once per device (every GPU holds its own copy of the
+// array at its own address).
+constexpr int kMaxDevices = 64;
+std::atomic<float*> g_scratch_addr[kMaxDevices];
+
+int static_scratch(const char* fn, float** out) {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return fail(PICO_ERR_LAUNCH, "%s: cannot tell the current device", fn);
+  float* p = g_scratch_addr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    const hipError_t e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(PICO_ERR_LAUNCH, "%s: hipGetSymbolAddress(scratch) failed on device %d: %s", fn, dev, hipGetErrorString(e));
+    g_scratch_addr[dev].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return PICO_OK;
+}
+
+}  // namespace
+
+extern "C" int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd,
+                                const void* dresidual, void* dx, void* dweight, int dweight_dtype, void* workspace,
+                                int64_t workspace_bytes, int64_t rows, int64_t hidden, int dtype, void* stream) {
+  return rmsnorm_bwd_impl("pico_rmsnorm_bwd", dy, x, weight, rstd, dresidual, dx, dweight, dweight_dtype,
+                          static_cast<float*>(workspace), workspace_bytes, rows, hidden, dtype,
+                          static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t pico_rmsnorm_bwd_static_max_bytes(void) {
+  return static_cast<int64_t>(kStaticScratchFloats * sizeof(float));
+}
+
+extern "C" int pico_rmsnorm_bwd_static(const void* dy, const void* x, const void* weight, const float* rstd,
+                                       const void* dresidual, void* dx, void* dweight, int dweight_dtype, int64_t rows,
+                                       int64_t hidden, int dtype, void* stream) {
+  const char* fn = "pico_rmsnorm_bwd_static";
+  if (int rc = check_common(fn, rows, hidden, dtype)) return rc;
+  const int64_t need = bwd_partial_bytes(rows, hidden, dtype);
+  if (need > pico_rmsnorm_bwd_static_max_bytes())
+    return fail(PICO_ERR_WORKSPACE, "%s: rows=%lld hidden=%lld need %lld bytes of partial sums, the static scratch "
+                "holds %lld; use pico_rmsnorm_bwd with a workspace", fn, static_cast<long long>(rows),
+                static_cast<long long>(hidden), static_cast<long long>(need),
+                static_cast<long long>(pico_rmsnorm_bwd_static_max_bytes()));
+  float* partial = nullptr;
+  if (int rc = static_scratch(fn, &partial)) return rc;
+  return rmsnorm_bwd_impl(fn, dy, x, weight, rstd, dresidual, dx, dweight, dweight_dtype, partial,
+                          pico_rmsnorm_bwd_static_max_bytes(), rows, hidden, dtype, static_cast<hipStream_t>(stream));
 }
