@@ -368,12 +368,19 @@ void launch_fwd(const void* x, const void* w, void* y, float* rstd, const void* 
 }
 
 template <typename T, int G, int NV>
-void launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx,
-                float* partial, int blocks, int64_t rows, int hidden, hipStream_t s) {
+int launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, const void* dres, void* dx,
+               float* partial, int blocks, int64_t rows, int hidden, hipStream_t s) {
   const size_t lds = (kBwdThreads / G > 1) ? static_cast<size_t>(hidden) * sizeof(float) : 0;
+  // the longest rows need the whole default LDS allowance for the dweight row plus the kernel's static 32 bytes
+  static std::atomic<bool> lds_reserved{false};
+  constexpr size_t kLdsMax = static_cast<size_t>(G) * NV * io<T>::kVec * sizeof(float) + 64;
+  if (kLdsMax > 48 * 1024 &&
+      !reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(&rmsnorm_bwd_kernel<T, G, NV>), kLdsMax))
+    return fail(PICO_ERR_LAUNCH, "pico_rmsnorm_bwd: cannot reserve %zu bytes of LDS", kLdsMax);
   hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, G, NV>), dim3(blocks), dim3(kBwdThreads), lds, s,
                      static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), rstd,
                      static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden);
+  return PICO_OK;
 }
 
 template <typename T>
@@ -409,8 +416,7 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
   {                                                                                \
     const int blocks = bwd_blocks(rows, kBwdThreads / G, hidden);                          \
     *blocks_out = blocks;                                                          \
-    launch_bwd<T, G, NV>(dy, x, w, rstd, dres, dx, partial, blocks, rows, hidden, s); \
-    return PICO_OK;                                                                \
+    return launch_bwd<T, G, NV>(dy, x, w, rstd, dres, dx, partial, blocks, rows, hidden, s); \
   }
 #define PICO_BWD_WAVE(NV)                                                                              \
   {                                                                                                    \
@@ -427,7 +433,7 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
                          rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
     return PICO_OK;                                                                                    \
   }
-  if (nv_wave && static_cast<size_t>(hidden) * 3 * sizeof(float) <= 65536) {
+  if (nv_wave) {   // rows of at most 64 x 8 vectors: (4 - 1) waves x hidden floats of LDS is at most 48 KiB
     switch (nv_wave) {
       case 1: PICO_BWD_WAVE(1);
       case 2: PICO_BWD_WAVE(2);
@@ -435,17 +441,12 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
       default: PICO_BWD_WAVE(8);
     }
   }
-  if (nv_wave) {
-    switch (nv_wave) {
-      case 1: PICO_BWD(64, 1);
-      case 2: PICO_BWD(64, 2);
-      case 4: PICO_BWD(64, 4);
-      default: PICO_BWD(64, 8);
-    }
-  }
-  switch (pick_nv((nvec + 255) / 256, 8)) {
+  // longer rows: one row per 256 threads, two rows per block.  The two groups add their shares of dweight to the
+  // block's LDS row with LDS atomics; two addends commute, so the sum does not depend on which arrives first.
+  switch (pick_nv((nvec + 255) / 256, 16)) {
     case 4: PICO_BWD(256, 4);
     case 8: PICO_BWD(256, 8);
+    case 16: PICO_BWD(256, 16);
     default: break;
   }
 #undef PICO_BWD_WAVE
@@ -460,8 +461,7 @@ int64_t bwd_partial_bytes(int64_t rows, int64_t hidden, int dtype) {
   const int nvec = static_cast<int>(hidden / vec);
   const int nv_wave = pick_nv((nvec + 63) / 64, 8);
   int gpb;
-  if (nv_wave && static_cast<size_t>(hidden) * 3 * sizeof(float) <= 65536) gpb = kBwdWaveThreads / kWave;
-  else if (nv_wave) gpb = kBwdThreads / 64;
+  if (nv_wave) gpb = kBwdWaveThreads / kWave;
   else gpb = kBwdThreads / 256;
   return static_cast<int64_t>(bwd_blocks(rows, gpb, static_cast<int>(hidden))) * hidden * static_cast<int64_t>(sizeof(float));
 }

@@ -35,7 +35,7 @@ def ops(device):
 
 
 # ------------------------------------------------------------------------------------ RMSNorm
-@pytest.mark.parametrize("rows,hidden", [(7, 576), (64, 2048), (33, 4096), (5, 8192), (3, 64), (0, 128)])
+@pytest.mark.parametrize("rows,hidden", [(7, 576), (64, 2048), (33, 4096), (5, 8192), (3, 64), (0, 128), (6, 16384), (9, 12288)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("cts", [True, False])
 def test_rmsnorm_fwd(ops, device, rows, hidden, dtype, cts):
@@ -65,7 +65,7 @@ def test_rmsnorm_fwd_residual(ops, device):
     assert maxabs(y, OL.rmsnorm(h, w.float(), 1e-5, cast_then_scale=False)) <= 2e-2
 
 
-@pytest.mark.parametrize("rows,hidden", [(7, 576), (300, 2048), (1030, 1024), (33, 4096), (5, 8192), (0, 64)])
+@pytest.mark.parametrize("rows,hidden", [(7, 576), (300, 2048), (1030, 1024), (33, 4096), (5, 8192), (0, 64), (6, 16384), (9, 12288)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_rmsnorm_bwd(ops, device, rows, hidden, dtype):
     x, dy = rnd(rows, hidden, seed=6, dtype=dtype), rnd(rows, hidden, seed=7, dtype=dtype)
