@@ -54,9 +54,10 @@ def parse():
     ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B- and Llama-2-7B-shaped training steps")
     ap.add_argument("--train-step", choices=["smollm_1p7b", "llama2_7b"], default=None,
                     help="run only that training step (for a kernel trace of it) and print its figures")
-    ap.add_argument("--probe", action="store_true",
+    ap.add_argument("--probe", nargs="?", const="configs1", default=None, choices=["configs1", "configs4"],
                     help="counter probe: a few launches of a plain copy of known size and of each attention kernel "
-                         "at the bench shape, nothing else (for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)")
+                         "at the bench shape (configs1) or at configs[4]'s shape (rank 7 of 8, head_dim 128), nothing else "
+                         "(for rocprofv3 --pmc)")
     return ap.parse_args()
 
 
@@ -105,23 +106,17 @@ class RingBench:
             q, k, v, _, out, _, _ = self._views(r)
             self.ops.attn_fwd(q, k, v, self.scale, True, r * self.Sc, out=out, lse=self.lse[r])
 
-    def backward_kernels_only(self):
-        for r in range(self.W):
-            q, k, v, do, out, dk, dv = self._views(r)
-            self.ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, self.dq_acc[r],
-                              dk, dv, dkv_accumulate=True)
-
     def backward(self):
-        self.dk_acc.zero_()
-        self.dv_acc.zero_()
+        """One launch pair (dQ, dK/dV) per rank, last rank first: its dK/dV launch covers every chunk and writes where
+        the earlier ranks add, so no accumulator is cleared; delta = sum_d dO * O is computed inside the dQ kernel; dq is
+        written in bf16 directly (a rank owns its query chunk), dk / dv are summed over the ranks in fp32."""
         ops = self.ops
-        for r in range(self.W):
+        for r in reversed(range(self.W)):
             q, k, v, do, out, dk, dv = self._views(r)
-            delta = ops.attn_bwd_preprocess(do, out, delta=self.delta[r])
-            ops.attn_bwd(do, q, k, v, self.lse[r], delta, self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
-                         dkv_accumulate=True)
+            dq = self.dq_b[:, :, r * self.Sc:(r + 1) * self.Sc]
+            ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, dq, dk, dv,
+                         dkv_accumulate=r != self.W - 1, out=out)
         # hand the gradients back in the dtype of the inputs (autograd's cast in the reference)
-        self.dq = [ops.convert_f32(self.dq_acc[r], self.torch.bfloat16) for r in range(self.W)]
         self.dk = ops.convert_f32(self.dk_acc, self.torch.bfloat16)
         self.dv = ops.convert_f32(self.dv_acc, self.torch.bfloat16)
 
@@ -137,6 +132,38 @@ class RingBench:
         delta = ops.attn_bwd_preprocess(do, out, delta=self.delta[r])
         ops.attn_bwd(do, q, k, v, self.lse[r], delta, self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
                      dkv_accumulate=True)
+
+    def step_ranks_parallel(self):
+        """One launch per rank and direction, like step(), but the ranks' launches are independent branches: rank r's
+        forward, delta pre-pass and dQ kernel run on stream r, the dK/dV launches (which add into shared chunks) follow
+        each other on the calling stream, last rank first -- its launch covers every chunk and writes instead of adding,
+        so no accumulator is cleared.  Recorded into a graph the streams become parallel branches of the graph."""
+        torch, ops = self.torch, self.ops
+        cur = torch.cuda.current_stream()
+        if not hasattr(self, "_branch"):
+            self._branch = [torch.cuda.Stream() for _ in range(self.W)]      # default priority
+        ready = []
+        for r, st in enumerate(self._branch):
+            st.wait_stream(cur)
+            with torch.cuda.stream(st):
+                q, k, v, do, out, dk, dv = self._views(r)
+                ops.attn_fwd(q, k, v, self.scale, True, r * self.Sc, out=out, lse=self.lse[r])
+                ops.attn_bwd_preprocess(do, out, delta=self.delta[r])
+                ev = torch.cuda.Event()
+                ev.record(st)
+                ready.append(ev)
+                ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, self.dq_acc[r],
+                             want_dkv=False)
+        for r in reversed(range(self.W)):
+            cur.wait_event(ready[r])
+            q, k, v, do, out, dk, dv = self._views(r)
+            ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, None, dk, dv,
+                         dkv_accumulate=r != self.W - 1, want_dq=False)
+        for st in self._branch:
+            cur.wait_stream(st)
+        self.dq = [ops.convert_f32(self.dq_acc[r], torch.bfloat16) for r in range(self.W)]
+        self.dk = ops.convert_f32(self.dk_acc, torch.bfloat16)
+        self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
 
     # -- all four ranks in one launch per direction (q_offset 0 over the whole sequence)
     def forward_batched(self):
@@ -505,6 +532,27 @@ def main():
     if args.train_step:
         print(json.dumps({args.train_step + "_train_step": train_step_extra(torch, args.train_step, steps=4, warmup=2)}))
         return
+    if args.probe == "configs4":
+        W, Sc, Hq, Hkv, D, r = 8, 4096, 32, 8, 128, 7
+        scale = 1.0 / math.sqrt(D)
+        g = torch.Generator().manual_seed(0)
+        q = (torch.randn(1, Hq, Sc, D, generator=g) * scale).to(torch.bfloat16).cuda()
+        k, v = (torch.randn(1, Hkv, W * Sc, D, generator=g).to(torch.bfloat16).cuda() for _ in range(2))
+        do = torch.randn(1, Hq, Sc, D, generator=g).to(torch.bfloat16).cuda()
+        out, dq, dk, dv = torch.empty_like(q), torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        lse = torch.empty(1, Hq, Sc, dtype=torch.float32, device="cuda")
+        src = torch.randn(16, 1024, 1024, dtype=torch.float32, device="cuda").view(1, 16, 1024, 1024)
+        for _ in range(3):
+            ops.convert_f32(src, torch.float32)
+        for _ in range(3):
+            ops.attn_fwd(q, k, v, scale, True, r * Sc, out=out, lse=lse)
+            delta = ops.attn_bwd_preprocess(do, out)
+            ops.attn_bwd(do, q, k, v, lse, delta, scale, True, r * Sc, None, dk, dv, want_dq=False)
+            ops.attn_bwd(do, q, k, v, lse, delta, scale, True, r * Sc, dq, want_dkv=False)
+        torch.cuda.synchronize()
+        print(json.dumps({"probe": "convert_kernel<float> copies 67108864 B in and out per launch; attention kernels at configs[4] "
+                                   "(rank 7 of 8: 4096 queries x 32768 keys, GQA 32/8, head_dim 128)"}))
+        return
     rb = RingBench(torch, ops)
     if args.probe:
         # plain copy of 64 MiB fp32 (read 64 MiB, write 64 MiB) as the scale for the HBM counters
@@ -581,13 +629,24 @@ def main():
         extras["attn_fwd_kernel"] = {"TFLOP/s": round(fwd_flops / (ms_fwd * 1e-3) / 1e12, 2), "us_per_launch": round(ms_fwd * 1e3, 2),
                                      "frac_of_mfma_peak": round(fwd_flops / (ms_fwd * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
         ms_rank, _ = graph_time(torch, rb.step, max(args.steps // 4, 10))
-        extras["one_launch_per_rank"] = {"TFLOP/s": round(total_flops / (ms_rank * 1e-3) / 1e12, 2), "ms_per_step": round(ms_rank, 4)}
+        extras["one_launch_per_rank"] = {"TFLOP/s": round(total_flops / (ms_rank * 1e-3) / 1e12, 2), "ms_per_step": round(ms_rank, 4),
+                                         "frac_of_mfma_peak": round(total_flops / (ms_rank * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                         "schedule": "ranks one after another on one stream"}
+        ms_par, _ = graph_time(torch, rb.step_ranks_parallel, max(args.steps // 4, 10))
+        extras["one_launch_per_rank_parallel_branches"] = {
+            "TFLOP/s": round(total_flops / (ms_par * 1e-3) / 1e12, 2), "ms_per_step": round(ms_par, 4),
+            "frac_of_mfma_peak": round(total_flops / (ms_par * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "schedule": "rank r's forward, delta and dQ on graph branch r; the dK/dV launches in sequence, last rank first"}
         ms_r3, _ = graph_time(torch, lambda: rb.step_one_rank(3), max(args.steps // 10, 10), per_graph=10)
         r3_flops = total_flops * 3.5 / 8.0   # 1 causal + 3 dense chunk-blocks of the 8 block-equivalents of all ranks
         extras["rank3_of_4_alone"] = {"TFLOP/s": round(r3_flops / (ms_r3 * 1e-3) / 1e12, 2), "us_per_step": round(ms_r3 * 1e3, 2),
-                                      "flops": r3_flops}
+                                      "flops": r3_flops,
+                                      "frac_of_mfma_peak": round(r3_flops / (ms_r3 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                      "schedule": "the last rank's share alone: 256 queries of every head over chunks 0..3"}
         ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
-        extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4)}
+        extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4),
+                                              "frac_of_mfma_peak": round(total_flops / (ms_ring * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+                                              "schedule": "the reference's shape: block + fused merge per ring step, ranks and steps in sequence"}
         extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
         extras["configs4_long_context_rank7_of_8"] = long_context_extra(torch, ops)
         if not args.no_train:

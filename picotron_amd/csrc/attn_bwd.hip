@@ -67,6 +67,23 @@ constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 #ifndef PICO_DKDV_PRIO
 #define PICO_DKDV_PRIO 1
 #endif
+// The scores are needed as exp2(s * sm_scale * log2e - lse * log2e).  With PICO_PRESCALE the factor is folded into one
+// bf16 operand of the S product once per kernel (K fragments in the dK/dV kernel, Q fragments in the dQ kernel) and
+// -lse * log2e is what the S accumulator starts from, so the exponent comes out of the MFMA and the multiply-add in
+// front of every v_exp_f32 disappears (one of about seven vector instructions per score).  The scaled operand is
+// rounded to bf16 once more: an error of 2^-9 relative per element, i.e. of the size of the inputs' own rounding.
+#ifndef PICO_PRESCALE
+#define PICO_PRESCALE 1
+#endif
+constexpr bool kPrescale = PICO_PRESCALE != 0;
+
+template <int N>
+__device__ __forceinline__ void scale_fragments(bf16x8 (&f)[N], float c) {
+#pragma unroll
+  for (int s = 0; s < N; ++s)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[s][e] = static_cast<__bf16>(static_cast<float>(f[s][e]) * c);
+}
 
 template <int D>
 struct KvCfg {
@@ -126,6 +143,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
     kt.fragments(region, lane, kf);
     vt.fragments(region, lane, vf);
+    if constexpr (kPrescale) scale_fragments(kf, c);   // kf feeds the S product only (dK comes from Q^T dS)
   }
 
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
@@ -216,7 +234,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     if (tid < BM) {
       // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
       const bool live = static_cast<uint32_t>(tid) * 4u < cur.rows_left && lreg != -INFINITY;
-      sL[tid] = live ? lreg * kLog2e : INFINITY;
+      // (with kPrescale the value is the S accumulator's start, so it is stored negated)
+      sL[tid] = kPrescale ? (live ? -lreg * kLog2e : -INFINITY) : (live ? lreg * kLog2e : INFINITY);
       sDelta[tid] = -dreg;   // stored negated: it is loaded straight into the dP accumulator (0 past Sq)
     }
   };
@@ -254,8 +273,10 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
+        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (kPrescale) s4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) { s_acc[4 * j + t] = 0.f; dp_acc[4 * j + t] = d4[t]; }
+        for (int t = 0; t < 4; ++t) { s_acc[4 * j + t] = s4[t]; dp_acc[4 * j + t] = d4[t]; }
       }
 #pragma unroll
       for (int s = 0; s < D / 16; ++s) {
@@ -273,11 +294,12 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       const int key_rel = kw0 + n - qs_pos - 4 * h;  // key is masked for row (8j + 4h + t) iff key_rel > 8j + t
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
+        f32x4 l4 = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (!kPrescale) l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const int i = 4 * j + t;
-          float pv = fast_exp2(s_acc[i] * c - l4[t]);
+          float pv = kPrescale ? fast_exp2(s_acc[i]) : fast_exp2(s_acc[i] * c - l4[t]);
           if constexpr (kMask) {
             if (key_rel > 8 * j + t) pv = 0.f;
           }
@@ -329,7 +351,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       auto softmax_part = [&](f32x16& s_acc, f32x16& dp_acc, const f32x4 (&l4)[4], int first, int count) {
 #pragma unroll
         for (int i = first; i < first + count; ++i) {
-          const float pv = fast_exp2(s_acc[i] * c - l4[i / 4][i % 4]);
+          const float pv = kPrescale ? fast_exp2(s_acc[i]) : fast_exp2(s_acc[i] * c - l4[i / 4][i % 4]);
           s_acc[i] = pv;
           dp_acc[i] = pv * dp_acc[i];
         }
@@ -343,13 +365,17 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
         // lse rows of sub-block 0 are fetched a slot ahead of the elements that need them (kPer elements per slot)
         constexpr int kPer = 16 / kPairs;
         f32x4 l4[4];
-        auto lse_row = [&](int r) { l4[r] = *reinterpret_cast<const f32x4*>(&sL[8 * r + 4 * h]); };
+        auto lse_row = [&](int r) {
+          if constexpr (!kPrescale) l4[r] = *reinterpret_cast<const f32x4*>(&sL[8 * r + 4 * h]);
+        };
         lse_row(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 + 8 * j + 4 * h]);
+          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (kPrescale) s4 = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * j + 4 * h]);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) { s1[4 * j + t] = 0.f; d1[4 * j + t] = d4[t]; }
+          for (int t = 0; t < 4; ++t) { s1[4 * j + t] = s4[t]; d1[4 * j + t] = d4[t]; }
         }
         bf16x8 qa[kPairs], da[kPairs];
         auto fetch = [&](int j) {
@@ -374,7 +400,9 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       {
         constexpr int kPer = 16 / kSlots;
         f32x4 l4[4];
-        auto lse_row = [&](int r) { l4[r] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * r + 4 * h]); };
+        auto lse_row = [&](int r) {
+          if constexpr (!kPrescale) l4[r] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * r + 4 * h]);
+        };
         lse_row(0);
         bf16x8 dof[kSlots], qf[kSlots];
         auto fetch = [&](int idx) {
@@ -483,6 +511,10 @@ template <> struct KvKernel<128> { static constexpr auto fn = &attn_bwd_dkdv_ker
 // =====================================================================================  dQ
 // KS > 1: KS waves share the same 32 queries and each takes one 64-key step of every staged tile (see the forward
 // kernel); their dQ partial sums meet in LDS at the end.
+// workgroups of 256 queries (8 waves) a launch must have before that size is used
+#ifndef PICO_DQ_NW8_MIN
+#define PICO_DQ_NW8_MIN 512
+#endif
 template <int D, int NW, int KT, int KS = 1>
 struct DqCfg {
   static constexpr int kThreads = 64 * NW;
@@ -521,6 +553,8 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
   const int n = lane % 32, h = lane / 32;
   const int qw = wave % C::kQWaves, ks = wave / C::kQWaves;   // which queries, which 64-key step of a staged tile
   const float c = a.sm_scale * kLog2e;
+  // (at head_dim 128 the kernel has no registers left for the accumulator's 16-register start value)
+  constexpr bool kPre = kPrescale && D <= 64;
 
   const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
   const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
@@ -551,6 +585,7 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
     unsigned char* region = smem_raw + wave * WaveTile<D>::kRegionBytes;
     qt.fragments(region, lane, qf);
     dt.fragments(region, lane, dof);
+    if constexpr (kPre) scale_fragments(qf, c);   // qf feeds the S product only
     if constexpr (kDelta) {
       // delta = sum_d dO * O of the lane's row (context_parallel.py:145): each half of the wave holds half of the
       // row's columns in its fragments; the dK/dV kernel, launched after this one, reads the result from memory
@@ -652,8 +687,9 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
       if constexpr (KS == 1) __builtin_amdgcn_iglp_opt(0);
 #pragma unroll
       for (int mb = 0; mb < BN / 32; ++mb) {
+        // dP - delta comes out of the MFMA, and with kPre so does the exponent s * c - lse * log2e
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = 0.f; dp_acc[mb][i] = -delta; }  // dP - delta comes out of the MFMA
+        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = kPre ? -lse2 : 0.f; dp_acc[mb][i] = -delta; }
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) {
           const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
@@ -680,7 +716,7 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
       for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const float pv = fast_exp2(s_acc[mb][i] * c - lse2);
+          const float pv = kPre ? fast_exp2(s_acc[mb][i]) : fast_exp2(s_acc[mb][i] * c - lse2);
           dp_acc[mb][i] = pv * dp_acc[mb][i];
         }
       // ---- dQ^T[d][query] += K^T[d][key] dS^T[key][query]
@@ -904,7 +940,7 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     if (desc->D == 64) {
       auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
-      if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
+      if (groups(256) >= PICO_DQ_NW8_MIN) rc = launch_dq<64, 8, 64>(p, s);
       else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
       else rc = launch_dq<64, 4, 128, 2>(p, s);   // few waves in all: two waves per 32 queries, 64 keys of every 128 each
     } else {

@@ -70,6 +70,10 @@ struct FwdCfg {
 #ifndef PICO_FWD_KS
 #define PICO_FWD_KS 2
 #endif
+// workgroups of 256 queries (8 waves) a launch must have before that size is used
+#ifndef PICO_FWD_NW8_MIN
+#define PICO_FWD_NW8_MIN 512
+#endif
 #ifndef PICO_FWD_ATTR
 #define PICO_FWD_ATTR
 #endif
@@ -485,7 +489,7 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
   if (desc->D == 64) {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
-    if (groups(256) >= 512) rc = launch<PICO_FWD_CFG64>(p, s);
+    if (groups(256) >= PICO_FWD_NW8_MIN) rc = launch<PICO_FWD_CFG64>(p, s);
     else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
     else rc = launch<64, 1, 4, 128, PICO_FWD_KS>(p, s);   // few waves in all: two waves per 32 queries, 64 keys of every 128 each
   } else {
