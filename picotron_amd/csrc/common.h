@@ -66,6 +66,14 @@ template <> struct io<__bf16> {
     for (int i = 0; i < 4; ++i) raw[i] = pack_bf16x2(in[2 * i], in[2 * i + 1]);
     *reinterpret_cast<u32x4*>(p) = raw;
   }
+  // streaming (non-temporal) store: for data that nothing on the GPU reads back soon, or that is so large that keeping
+  // it in the caches only evicts what is still needed
+  static __device__ __forceinline__ void store_stream(void* p, const float (&in)[8]) {
+    u32x4 raw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = pack_bf16x2(in[2 * i], in[2 * i + 1]);
+    __builtin_nontemporal_store(raw, reinterpret_cast<u32x4*>(p));
+  }
   static __device__ __forceinline__ float round(float v) {
     return bf16_bits_to_float(float_to_bf16_bits(v));
   }
@@ -83,8 +91,21 @@ template <> struct io<float> {
     for (int i = 0; i < 4; ++i) raw[i] = in[i];
     *reinterpret_cast<f32x4*>(p) = raw;
   }
+  static __device__ __forceinline__ void store_stream(void* p, const float (&in)[4]) {
+    f32x4 raw;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) raw[i] = in[i];
+    __builtin_nontemporal_store(raw, reinterpret_cast<f32x4*>(p));
+  }
   static __device__ __forceinline__ float round(float v) { return v; }
 };
+
+// store<kStream>: picks the streaming form at compile time
+template <typename T, bool kStream, int N>
+__device__ __forceinline__ void store_as(void* p, const float (&in)[N]) {
+  if constexpr (kStream) io<T>::store_stream(p, in);
+  else io<T>::store(p, in);
+}
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 

@@ -12,6 +12,24 @@ static __device__ __align__(256) float scratch[kStaticScratchFloats];
 namespace pico {
 namespace {
 
+// which outputs leave with streaming stores (measured per kernel, see the bandwidth table of the bench)
+#ifndef PICO_NT_NORM_FWD
+#define PICO_NT_NORM_FWD 1
+#endif
+#ifndef PICO_NT_NORM_BWD
+#define PICO_NT_NORM_BWD 0
+#endif
+// read-once inputs fetched with the streaming hint
+#ifndef PICO_NT_NORM_LOADS
+#define PICO_NT_NORM_LOADS 1
+#endif
+__device__ __forceinline__ u32x4 load_raw(const void* p) {
+#if PICO_NT_NORM_LOADS
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#else
+  return *reinterpret_cast<const u32x4*>(p);
+#endif
+}
 constexpr int kFwdThreads = 256;
 constexpr int kBwdThreads = 512;
 constexpr int kMaxBwdBlocks = 512;   // rows of the dweight workspace
@@ -62,7 +80,7 @@ __global__ __launch_bounds__(kFwdThreads) void rmsnorm_fwd_kernel(
         io<T>::load(res_in + row * hidden + v * V, r);
 #pragma unroll
         for (int e = 0; e < V; ++e) vals[j][e] += r[e];
-        if (res_out != nullptr) io<T>::store(res_out + row * hidden + v * V, vals[j]);
+        if (res_out != nullptr) store_as<T, PICO_NT_NORM_FWD != 0>(res_out + row * hidden + v * V, vals[j]);
       }
 #pragma unroll
       for (int e = 0; e < V; ++e) ss += vals[j][e] * vals[j][e];
@@ -82,7 +100,7 @@ __global__ __launch_bounds__(kFwdThreads) void rmsnorm_fwd_kernel(
         const float n = vals[j][e] * r;
         o[e] = cast_then_scale ? io<T>::round(n) * wv[e] : n * wv[e];
       }
-      io<T>::store(y + row * hidden + v * V, o);
+      store_as<T, PICO_NT_NORM_FWD != 0>(y + row * hidden + v * V, o);
     }
   }
 }
@@ -151,7 +169,7 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
 #pragma unroll
           for (int e = 0; e < V; ++e) o[e] += dr[e];
         }
-        io<T>::store(dx + row * hidden + v * V, o);
+        store_as<T, PICO_NT_NORM_BWD != 0>(dx + row * hidden + v * V, o);
       }
     }
   }
@@ -212,9 +230,9 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
     for (int j = 0; j < NV; ++j) {
       const int v = t + j * kWave;
       const int vc = v < nvec ? v : 0;
-      xr[j] = *reinterpret_cast<const u32x4*>(x + r * hidden + vc * V);
-      dr[j] = *reinterpret_cast<const u32x4*>(dy + r * hidden + vc * V);
-      if constexpr (kRes) rr[j] = *reinterpret_cast<const u32x4*>(dres + r * hidden + vc * V);
+      xr[j] = load_raw(x + r * hidden + vc * V);
+      dr[j] = load_raw(dy + r * hidden + vc * V);
+      if constexpr (kRes) rr[j] = load_raw(dres + r * hidden + vc * V);
     }
     rs = rstd[r];
   };
@@ -264,7 +282,7 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
 #pragma unroll
           for (int e = 0; e < V; ++e) o[e] += rv[e];
         }
-        io<T>::store(dx + row * hidden + v * V, o);
+        store_as<T, PICO_NT_NORM_BWD != 0>(dx + row * hidden + v * V, o);
       }
     }
   }
@@ -299,11 +317,15 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
 }
 
 // dweight[c] = sum_p partial[p][c]; 32 columns x 32 slices per block, every thread's loads issued together.
-constexpr int kReduceCols = 32;
+#ifndef PICO_NORM_REDUCE_COLS
+#define PICO_NORM_REDUCE_COLS 32
+#endif
+constexpr int kReduceCols = PICO_NORM_REDUCE_COLS;
+constexpr int kReduceSlices = 1024 / kReduceCols;
 template <typename TW>
-__global__ __launch_bounds__(kReduceCols * 32) void rmsnorm_dw_reduce_kernel(
+__global__ __launch_bounds__(1024) void rmsnorm_dw_reduce_kernel(
     const float* __restrict__ partial, TW* __restrict__ dweight, int nparts, int hidden) {
-  constexpr int kSlices = 32, kUnroll = 16;
+  constexpr int kSlices = kReduceSlices, kUnroll = 512 / kSlices;
   __shared__ float red[kSlices][kReduceCols + 1];
   const int c = threadIdx.x % kReduceCols;
   const int col = blockIdx.x * kReduceCols + c;
@@ -332,7 +354,7 @@ __global__ __launch_bounds__(kReduceCols * 32) void rmsnorm_dw_reduce_kernel(
 }
 
 void launch_dw_reduce(const float* partial, void* dweight, int dweight_dtype, int nparts, int hidden, hipStream_t s) {
-  const dim3 grid(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)), block(kReduceCols * 32);
+  const dim3 grid(static_cast<unsigned>((hidden + kReduceCols - 1) / kReduceCols)), block(1024);
   if (dweight_dtype == PICO_BF16)
     hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<__bf16>, grid, block, 0, s, partial, static_cast<__bf16*>(dweight), nparts, hidden);
   else

@@ -3,6 +3,17 @@
 // lanes touch consecutive memory for the layout at hand.
 #include "common.h"
 
+// which outputs leave with streaming stores (measured per kernel, see the bandwidth table of the bench)
+#ifndef PICO_NT_ROPE
+#define PICO_NT_ROPE 0
+#endif
+#ifndef PICO_NT_SWIGLU_FWD
+#define PICO_NT_SWIGLU_FWD 0
+#endif
+#ifndef PICO_NT_SWIGLU_BWD
+#define PICO_NT_SWIGLU_BWD 1
+#endif
+
 namespace pico {
 namespace {
 
@@ -66,8 +77,8 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(
     olo[e] = lo[e] * c[e] - hi[e] * sg;
     ohi[e] = hi[e] * c[e] + lo[e] * sg;
   }
-  io<T>::store(yp, olo);
-  io<T>::store(yp + half, ohi);
+  store_as<T, PICO_NT_ROPE != 0>(yp, olo);
+  store_as<T, PICO_NT_ROPE != 0>(yp + half, ohi);
 }
 
 // ---------------------------------------------------------------------------------- SwiGLU
@@ -87,7 +98,7 @@ __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const T* __restric
   io<T>::load(up + r * uld + c, u);
 #pragma unroll
   for (int e = 0; e < V; ++e) o[e] = g[e] * sigmoidf_fast(g[e]) * u[e];
-  io<T>::store(y + r * yld + c, o);
+  store_as<T, PICO_NT_SWIGLU_FWD != 0>(y + r * yld + c, o);
 }
 
 template <typename T>
@@ -112,8 +123,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const T* __restric
     og[e] = d[e] * u[e] * (sg + silu * (1.f - sg));
     ou[e] = d[e] * silu;
   }
-  io<T>::store(dgate + r * dgld + c, og);
-  io<T>::store(dup + r * duld + c, ou);
+  store_as<T, PICO_NT_SWIGLU_BWD != 0>(dgate + r * dgld + c, og);
+  store_as<T, PICO_NT_SWIGLU_BWD != 0>(dup + r * duld + c, ou);
 }
 
 // ---------------------------------------------------------------------------------- lse merge
