@@ -60,6 +60,15 @@ template <> struct io<__bf16> {
       out[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
     }
   }
+  // streaming load: for inputs a kernel reads once (they need not stay in the caches)
+  static __device__ __forceinline__ void load_stream(const void* p, float (&out)[8]) {
+    u32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      out[2 * i] = __uint_as_float(raw[i] << 16);
+      out[2 * i + 1] = __uint_as_float(raw[i] & 0xffff0000u);
+    }
+  }
   static __device__ __forceinline__ void store(void* p, const float (&in)[8]) {
     u32x4 raw;
 #pragma unroll
@@ -85,6 +94,11 @@ template <> struct io<float> {
 #pragma unroll
     for (int i = 0; i < 4; ++i) out[i] = raw[i];
   }
+  static __device__ __forceinline__ void load_stream(const void* p, float (&out)[4]) {
+    f32x4 raw = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out[i] = raw[i];
+  }
   static __device__ __forceinline__ void store(void* p, const float (&in)[4]) {
     f32x4 raw;
 #pragma unroll
@@ -100,6 +114,11 @@ template <> struct io<float> {
   static __device__ __forceinline__ float round(float v) { return v; }
 };
 
+template <typename T, bool kStream, int N>
+__device__ __forceinline__ void load_as(const void* p, float (&out)[N]) {
+  if constexpr (kStream) io<T>::load_stream(p, out);
+  else io<T>::load(p, out);
+}
 // store<kStream>: picks the streaming form at compile time
 template <typename T, bool kStream, int N>
 __device__ __forceinline__ void store_as(void* p, const float (&in)[N]) {

@@ -19,6 +19,9 @@ namespace {
 #ifndef PICO_NT_NORM_BWD
 #define PICO_NT_NORM_BWD 0
 #endif
+#ifndef PICO_NT_NORM_FWD_LOADS
+#define PICO_NT_NORM_FWD_LOADS 0
+#endif
 // read-once inputs fetched with the streaming hint
 #ifndef PICO_NT_NORM_LOADS
 #define PICO_NT_NORM_LOADS 1
@@ -74,10 +77,10 @@ __global__ __launch_bounds__(kFwdThreads) void rmsnorm_fwd_kernel(
   for (int j = 0; j < NV; ++j) {
     const int v = t + j * G;
     if (v < nvec) {
-      io<T>::load(xr + v * V, vals[j]);
+      load_as<T, PICO_NT_NORM_FWD_LOADS != 0>(xr + v * V, vals[j]);
       if (res_in != nullptr) {
         float r[V];
-        io<T>::load(res_in + row * hidden + v * V, r);
+        load_as<T, PICO_NT_NORM_FWD_LOADS != 0>(res_in + row * hidden + v * V, r);
 #pragma unroll
         for (int e = 0; e < V; ++e) vals[j][e] += r[e];
         if (res_out != nullptr) store_as<T, PICO_NT_NORM_FWD != 0>(res_out + row * hidden + v * V, vals[j]);

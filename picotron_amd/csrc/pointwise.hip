@@ -10,6 +10,12 @@
 #ifndef PICO_NT_SWIGLU_FWD
 #define PICO_NT_SWIGLU_FWD 0
 #endif
+#ifndef PICO_NT_ROPE_LOADS
+#define PICO_NT_ROPE_LOADS 0
+#endif
+#ifndef PICO_NT_SWIGLU_LOADS
+#define PICO_NT_SWIGLU_LOADS 0
+#endif
 #ifndef PICO_NT_SWIGLU_BWD
 #define PICO_NT_SWIGLU_BWD 1
 #endif
@@ -47,8 +53,8 @@ __global__ __launch_bounds__(kThreads) void rope_kernel(
   const T* xp = x + b * xsb + h * xsh + s * xss + v * V;
   T* yp = y + b * ysb + h * ysh + s * yss + v * V;
   float lo[V], hi[V], c[V], sn[V];
-  io<T>::load(xp, lo);
-  io<T>::load(xp + half, hi);
+  load_as<T, PICO_NT_ROPE_LOADS != 0>(xp, lo);
+  load_as<T, PICO_NT_ROPE_LOADS != 0>(xp + half, hi);
   const int64_t trow = (pos_offset + s) * table_ld + v * V;
   if constexpr (io<TT>::kVec == V) {
     io<TT>::load(cos_t + trow, c);
@@ -94,8 +100,8 @@ __global__ __launch_bounds__(kThreads) void swiglu_fwd_kernel(const T* __restric
   const int64_t r = idx / vpr;
   const int64_t c = (idx % vpr) * V;
   float g[V], u[V], o[V];
-  io<T>::load(gate + r * gld + c, g);
-  io<T>::load(up + r * uld + c, u);
+  load_as<T, PICO_NT_SWIGLU_LOADS != 0>(gate + r * gld + c, g);
+  load_as<T, PICO_NT_SWIGLU_LOADS != 0>(up + r * uld + c, u);
 #pragma unroll
   for (int e = 0; e < V; ++e) o[e] = g[e] * sigmoidf_fast(g[e]) * u[e];
   store_as<T, PICO_NT_SWIGLU_FWD != 0>(y + r * yld + c, o);
@@ -113,9 +119,9 @@ __global__ __launch_bounds__(kThreads) void swiglu_bwd_kernel(const T* __restric
   const int64_t r = idx / vpr;
   const int64_t c = (idx % vpr) * V;
   float d[V], g[V], u[V], og[V], ou[V];
-  io<T>::load(dy + r * dyld + c, d);
-  io<T>::load(gate + r * gld + c, g);
-  io<T>::load(up + r * uld + c, u);
+  load_as<T, PICO_NT_SWIGLU_LOADS != 0>(dy + r * dyld + c, d);
+  load_as<T, PICO_NT_SWIGLU_LOADS != 0>(gate + r * gld + c, g);
+  load_as<T, PICO_NT_SWIGLU_LOADS != 0>(up + r * uld + c, u);
 #pragma unroll
   for (int e = 0; e < V; ++e) {
     const float sg = sigmoidf_fast(g[e]);
