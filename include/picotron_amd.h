@@ -164,6 +164,29 @@ typedef struct pico_attn_desc {
 int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
                   void* out, float* lse, int out_dtype, int merge, void* stream);
 
+/* RoPE tables for the attention entry points that rotate inside the kernel: cos / sin [rows, >= D/2 columns]
+ * (get_cos_sin's tables, model.py:21-31: only the first D/2 columns are read), `pitch` elements between rows,
+ * dtype PICO_BF16 or PICO_F32, row index = absolute position.
+ */
+typedef struct pico_rope_tables {
+  const void* cos;
+  const void* sin;
+  int64_t pitch;
+  int32_t dtype;
+  int32_t rows;
+} pico_rope_tables;
+
+/* replaces: apply_rotary_pos_emb on q (model.py:131 / :136) followed by the attention forward (model.py:154-157),
+ * one chunk: q arrives UN-rotated and every query is rotated once, in the prologue of the workgroup that owns it
+ * (position = q_pos_offset + row; fp32 arithmetic, one rounding, as pico_rope); k_rot must already be rotated
+ * (pico_rope on k: a key tile is read by many workgroups, rotating it there would repeat the work).  If q_rot is
+ * given the rotated q is written there (bf16, its own b/h/s strides, unit D stride) for pico_attn_bwd_rope.
+ * Everything else as pico_attn_fwd with merge = 0.
+ */
+int pico_attn_fwd_rope(const pico_attn_desc* desc, const void* q, const void* k_rot, const void* v, void* out,
+                       float* lse, int out_dtype, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
+                       const int64_t* q_rot_stride, void* stream);
+
 /* replaces: D = sum(dO * O, dim=-1)  context_parallel.py:145.
  * delta: [B,Hq,Sq] fp32.  out is addressed by o_stride like dout and has dtype out_dtype.
  * If dq_acc is not NULL that [B,Hq,Sq,D] contiguous fp32 buffer is zeroed in the same pass (optional).
@@ -201,6 +224,19 @@ int pico_attn_bwd_fused(const pico_attn_desc* desc, const void* q, const void* k
                         void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate,
                         void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
                         void* stream);
+
+/* replaces: the backward of "rotate q and k, then attend" (autograd of model.py:131-137 + :154-157) for one chunk:
+ * pico_attn_bwd_fused on the ROTATED q and k (q_rot as written by pico_attn_fwd_rope, k_rot from pico_rope), with the
+ * backward of RoPE -- the rotation by the negative angle -- applied to dq and dk in the kernels' epilogues, in fp32,
+ * before their one rounding.  dq and dk are therefore gradients w.r.t. the UN-rotated q and k; no separate RoPE pass
+ * runs in the backward.  `out` is the bf16 forward output, `delta` an output as in pico_attn_bwd_fused; dq, dk and dv
+ * are all required and are written (not accumulated).  Positions: q_pos_offset + query row, k_pos_offset + key row.
+ */
+int pico_attn_bwd_rope(const pico_attn_desc* desc, const void* q_rot, const void* k_rot, const void* v,
+                       const void* dout, const void* out, const float* lse, float* delta,
+                       void* dq, const int64_t* dq_stride, int dq_dtype,
+                       void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
+                       const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset, void* stream);
 
 /* fp32 -> bf16/fp32 conversion with layout change: src [B,H,S,D] contiguous fp32,
  * dst addressed by dst_stride (b,h,s).  Used to hand dq_acc back in the dtype / layout of q.

@@ -24,6 +24,11 @@ class AttnDesc(Structure):
     ]
 
 
+class RopeTables(Structure):
+    """Mirror of ``pico_rope_tables``."""
+    _fields_ = [("cos", c_void_p), ("sin", c_void_p), ("pitch", c_int64), ("dtype", c_int32), ("rows", c_int32)]
+
+
 _P = c_void_p
 _I64 = c_int64
 SIGNATURES = {
@@ -39,6 +44,9 @@ SIGNATURES = {
     "pico_swiglu_bwd": (c_int, [_P] * 5 + [_I64] * 7 + [c_int, _P]),
     "pico_lse_merge": (c_int, [_P, _P, _P, _P, _I64, _I64, c_int, _P]),
     "pico_attn_fwd": (c_int, [POINTER(AttnDesc), _P, _P, _P, _P, _P, c_int, c_int, _P]),
+    "pico_attn_fwd_rope": (c_int, [POINTER(AttnDesc), _P, _P, _P, _P, _P, c_int, POINTER(RopeTables), c_int, _P, POINTER(c_int64), _P]),
+    "pico_attn_bwd_rope": (c_int, [POINTER(AttnDesc)] + [_P] * 5 + [_P, _P] + [_P, POINTER(c_int64), c_int, _P, _P, POINTER(c_int64), c_int,
+                                   POINTER(RopeTables), c_int, c_int, _P]),
     "pico_attn_bwd_preprocess": (c_int, [POINTER(AttnDesc), _P, _P, c_int, _P, _P, _P]),
     "pico_attn_bwd": (c_int, [POINTER(AttnDesc)] + [_P] * 6 + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int, _P]),
     "pico_attn_bwd_fused": (c_int, [POINTER(AttnDesc)] + [_P] * 5 + [c_int, _P, _P] + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int, _P]),

@@ -37,6 +37,7 @@ struct BwdParams {
   int pair_ktiles;  // dK/dV kernel: a workgroup takes key tile t and then tile n-1-t (equal work under a causal mask)
   int64_t dqs[3];  // element strides (b, h, s) of dq
   int64_t dks[3];  // element strides (b, h, s) of dk and dv
+  RopeArgs rope;   // rope.cos != nullptr: q and k are rotated tensors; dq and dk leave un-rotated (RoPE's backward)
 };
 
 // =====================================================================================  dK / dV
@@ -469,6 +470,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     const int row0 = key0 + 32 * wave;
     const int rows_live = a.Sk - row0;
     const int64_t off = b * p.dks[0] + hkv * p.dks[1] + static_cast<int64_t>(row0) * p.dks[2];
+    // gradient w.r.t. the un-rotated k: rotate the lane's row of dK back (linear, so the scale can follow)
+    if (p.rope.cos != nullptr) rope_unrotate_acc<D>(dk_acc, p.rope, n < rows_live ? p.rope.k_pos0 + row0 + n : 0, h);
     if (p.dkv_f32) {
       wave_store_rows<D, true>(region, dk_acc, a.sm_scale, static_cast<float*>(p.dk) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
       wave_store_rows<D, true>(region, dv_acc, 1.f, static_cast<float*>(p.dv) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
@@ -766,6 +769,7 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
     unsigned char* region = smem_raw + wave * kRowRegionBytes;
     const int row0 = q0 + qw * 32;
     const int64_t off = b * p.dqs[0] + hq * p.dqs[1] + static_cast<int64_t>(row0) * p.dqs[2];
+    if (p.rope.cos != nullptr) rope_unrotate_acc<D>(dq, p.rope, qlive ? p.rope.q_pos0 + qrow : 0, h);
     if (p.dq_f32)
       wave_store_rows<D, true>(region, dq, a.sm_scale, static_cast<float*>(p.dq) + off, p.dqs[2], a.Sq - row0, lane, p.dq_accumulate, false);
     else
@@ -884,7 +888,7 @@ namespace {
 int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
             const float* lse, const float* delta, const void* out, float* delta_w, void* dq, const int64_t* dq_stride,
             int dq_dtype, int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
-            int dkv_accumulate, void* stream) {
+            int dkv_accumulate, void* stream, const RopeArgs* rope = nullptr) {
   if ((dkv_dtype != PICO_BF16 && dkv_dtype != PICO_F32) || (dq_dtype != PICO_BF16 && dq_dtype != PICO_F32))
     return fail(PICO_ERR_DTYPE, "%s: gradient dtype codes %d / %d not supported", fn, dq_dtype, dkv_dtype);
   if ((dkv_accumulate && dkv_dtype != PICO_F32) || (dq_accumulate && dq_dtype != PICO_F32))
@@ -911,6 +915,7 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
   p.dkv_f32 = dkv_dtype == PICO_F32;
   p.dkv_accumulate = dkv_accumulate != 0;
   p.pair_ktiles = 0;
+  p.rope = rope ? *rope : RopeArgs{nullptr, nullptr, 0, 0, 0, 0};
   auto strides = [&](const int64_t* given, int heads, int seq, int64_t (&st)[3], int align) -> bool {
     if (given) {
       for (int i = 0; i < 3; ++i) {
@@ -987,4 +992,25 @@ extern "C" int pico_attn_bwd_fused(const pico_attn_desc* desc, const void* q, co
   }
   return run_bwd("pico_attn_bwd_fused", desc, q, k, v, dout, lse, delta, out, delta, dq, dq_stride, dq_dtype, dq_accumulate,
                  dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
+}
+
+extern "C" int pico_attn_bwd_rope(const pico_attn_desc* desc, const void* q_rot, const void* k_rot, const void* v,
+                                  const void* dout, const void* out, const float* lse, float* delta, void* dq,
+                                  const int64_t* dq_stride, int dq_dtype, void* dk, void* dv, const int64_t* dkv_stride,
+                                  int dkv_dtype, const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset,
+                                  void* stream) {
+  const char* fn = "pico_attn_bwd_rope";
+  if (int rc = check_attn_desc(fn, desc)) return rc;
+  if (desc->B == 0) return PICO_OK;
+  if (q_pos_offset < 0 || k_pos_offset < 0) return fail(PICO_ERR_SHAPE, "%s: position offsets must be >= 0", fn);
+  const int64_t last = (static_cast<int64_t>(q_pos_offset) + desc->Sq > static_cast<int64_t>(k_pos_offset) + desc->Sk
+                            ? static_cast<int64_t>(q_pos_offset) + desc->Sq
+                            : static_cast<int64_t>(k_pos_offset) + desc->Sk) - 1;
+  if (int rc = check_rope_tables(fn, rope, desc->D, last)) return rc;
+  if (!dq || !dk || !dv) return fail(PICO_ERR_NULL, "%s: dq, dk and dv are required", fn);
+  if (desc->Sq > 0 && (!out || !delta)) return fail(PICO_ERR_NULL, "%s: out and delta are required", fn);
+  const RopeArgs r{rope->cos, rope->sin, rope->pitch, rope->dtype == PICO_F32, q_pos_offset, k_pos_offset};
+  // the dQ kernel computes delta from the bf16 forward output in its prologue and runs before the dK/dV kernel
+  return run_bwd(fn, desc, q_rot, k_rot, v, dout, lse, delta, out, delta, dq, dq_stride, dq_dtype, 0, dk, dv, dkv_stride,
+                 dkv_dtype, 0, stream, &r);
 }

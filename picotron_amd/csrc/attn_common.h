@@ -191,6 +191,73 @@ __device__ __forceinline__ void wave_store_rows(unsigned char* region, const f32
   }
 }
 
+// ---- RoPE inside the attention kernels (non-interleaved: column d pairs with d + D/2; model.py:12-19).
+// Tables are [rows, >= D/2 columns] with `pitch` elements between rows, bf16 or fp32; row index = position.
+struct RopeArgs {
+  const void* cos;   // nullptr: no rotation
+  const void* sin;
+  int64_t pitch;
+  int f32;
+  int q_pos0, k_pos0;   // position of query row 0 / key row 0
+};
+// n (4 or 8) consecutive table entries starting at column `col` of row `pos`
+template <int N>
+__device__ __forceinline__ void rope_load(const RopeArgs& r, const void* table, int pos, int col, float (&out)[N]) {
+  if (r.f32) {
+    const float* t = static_cast<const float*>(table) + static_cast<int64_t>(pos) * r.pitch + col;
+#pragma unroll
+    for (int e = 0; e < N; e += 4) {
+      const f32x4 v = *reinterpret_cast<const f32x4*>(t + e);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) out[e + u] = v[u];
+    }
+  } else {
+    const __bf16* t = static_cast<const __bf16*>(table) + static_cast<int64_t>(pos) * r.pitch + col;
+#pragma unroll
+    for (int e = 0; e < N; e += 4) {
+      const u32x2 v = *reinterpret_cast<const u32x2*>(t + e);
+      out[e] = __uint_as_float(v[0] << 16);  out[e + 1] = __uint_as_float(v[0] & 0xffff0000u);
+      out[e + 2] = __uint_as_float(v[1] << 16);  out[e + 3] = __uint_as_float(v[1] & 0xffff0000u);
+    }
+  }
+}
+// Rotates a lane's operand fragments in place: fragment s holds columns 16 s + 8 h ..+7 of the lane's row, its partner
+// (column + D/2) is fragment s + D/32.  fp32 arithmetic, one rounding, the formula of the stand-alone kernel.
+template <int D>
+__device__ __forceinline__ void rope_rotate_fragments(bf16x8 (&f)[D / 16], const RopeArgs& r, int pos, int h) {
+#pragma unroll
+  for (int s = 0; s < D / 32; ++s) {
+    float c[8], sn[8];
+    rope_load<8>(r, r.cos, pos, 16 * s + 8 * h, c);
+    rope_load<8>(r, r.sin, pos, 16 * s + 8 * h, sn);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float lo = static_cast<float>(f[s][e]), hi = static_cast<float>(f[s + D / 32][e]);
+      f[s][e] = static_cast<__bf16>(lo * c[e] - hi * sn[e]);
+      f[s + D / 32][e] = static_cast<__bf16>(hi * c[e] + lo * sn[e]);
+    }
+  }
+}
+// Un-rotates (rotation by the negative angle: the backward of RoPE) a lane's row of a transposed-product accumulator:
+// registers 4j..4j+3 of block db hold columns 32 db + 8 j + 4 h ..+3; the partner of block db is block db + D/64.
+template <int D>
+__device__ __forceinline__ void rope_unrotate_acc(f32x16 (&acc)[D / 32], const RopeArgs& r, int pos, int h) {
+#pragma unroll
+  for (int db = 0; db < D / 64; ++db)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float c[4], sn[4];
+      rope_load<4>(r, r.cos, pos, 32 * db + 8 * j + 4 * h, c);
+      rope_load<4>(r, r.sin, pos, 32 * db + 8 * j + 4 * h, sn);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const float lo = acc[db][4 * j + t], hi = acc[db + D / 64][4 * j + t];
+        acc[db][4 * j + t] = lo * c[t] + hi * sn[t];
+        acc[db + D / 64][4 * j + t] = hi * c[t] - lo * sn[t];
+      }
+    }
+}
+
 struct AttnParams {
   const __bf16* q; const __bf16* k; const __bf16* v;
   int B, Hq, Hkv, Sq, Sk;
@@ -200,6 +267,8 @@ struct AttnParams {
 };
 
 int check_attn_desc(const char* fn, const pico_attn_desc* d);
+// tables usable for head_dim D and positions 0 .. last_pos?
+int check_rope_tables(const char* fn, const pico_rope_tables* t, int D, int64_t last_pos);
 AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, const void* v);
 
 }  // namespace pico

@@ -18,6 +18,9 @@ struct FwdParams {
   int out_f32;
   int merge;
   int pair_order;  // dispatch order of the query tiles, see the kernel
+  RopeArgs rope;   // rope.cos != nullptr: q arrives un-rotated and is rotated in the prologue (k is rotated already)
+  __bf16* q_rot;   // ... and, if given, the rotated q is written here for the backward
+  int64_t qrs[3];  // element strides (b, h, s) of q_rot
 };
 
 #ifndef PICO_FWD_KDEPTH
@@ -115,6 +118,16 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     WaveTile<D> qt;
     qt.issue(make_buffer(qbase + static_cast<int64_t>(row0) * a.qs[2], span_bytes(a.Sq - row0, a.qs[2], D)), a.qs[2], lane);
     qt.fragments(smem_raw + (wave * QB + qb) * WaveTile<D>::kRegionBytes, lane, qf[qb]);
+    if (p.rope.cos != nullptr) {
+      // RoPE on the wave's own queries, once per query in the whole launch (every query belongs to one wave)
+      const bool qlive = qrow[qb] < a.Sq;
+      rope_rotate_fragments<D>(qf[qb], p.rope, qlive ? p.rope.q_pos0 + qrow[qb] : 0, h);
+      if (p.q_rot != nullptr && qlive && (KS == 1 || ks == 0)) {
+        __bf16* dst = p.q_rot + b * p.qrs[0] + hq * p.qrs[1] + static_cast<int64_t>(qrow[qb]) * p.qrs[2];
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) *reinterpret_cast<bf16x8*>(dst + 16 * s + 8 * h) = qf[qb][s];
+      }
+    }
   }
 
   // ---- running state: m in the log2 domain (scores scaled by sm_scale*log2e), l split over the halves
@@ -446,6 +459,17 @@ int check_attn_desc(const char* fn, const pico_attn_desc* d) {
   return PICO_OK;
 }
 
+int check_rope_tables(const char* fn, const pico_rope_tables* t, int D, int64_t last_pos) {
+  if (!t || !t->cos || !t->sin) return fail(PICO_ERR_NULL, "%s: cos / sin tables are required", fn);
+  if (t->dtype != PICO_BF16 && t->dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: table dtype code %d not supported", fn, t->dtype);
+  if (t->pitch < D / 2 || t->pitch % 4 != 0 || !aligned16(t->cos) || !aligned16(t->sin) ||
+      (t->dtype == PICO_BF16 && t->pitch % 8 != 0))
+    return fail(PICO_ERR_STRIDE, "%s: table rows must hold D/2 columns, start 16-byte aligned and lie a multiple of 16 bytes apart", fn);
+  if (last_pos >= t->rows) return fail(PICO_ERR_SHAPE, "%s: positions up to %lld needed, the tables have %d rows", fn,
+                                       static_cast<long long>(last_pos), t->rows);
+  return PICO_OK;
+}
+
 AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, const void* v) {
   AttnParams a;
   a.q = static_cast<const __bf16*>(q);
@@ -465,23 +489,43 @@ AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, co
 
 using namespace pico;
 
-extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, void* out,
-                             float* lse, int out_dtype, int merge, void* stream) {
-  if (int rc = check_attn_desc("pico_attn_fwd", desc)) return rc;
+namespace {
+
+int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const void* k, const void* v, void* out, float* lse,
+            int out_dtype, int merge, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
+            const int64_t* q_rot_stride, void* stream) {
+  if (int rc = check_attn_desc(fn, desc)) return rc;
   if (out_dtype != PICO_BF16 && out_dtype != PICO_F32)
-    return fail(PICO_ERR_DTYPE, "pico_attn_fwd: out dtype code %d not supported", out_dtype);
-  if (merge && out_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "pico_attn_fwd: merge needs an fp32 running out");
+    return fail(PICO_ERR_DTYPE, "%s: out dtype code %d not supported", fn, out_dtype);
+  if (merge && out_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: merge needs an fp32 running out", fn);
   if (desc->B == 0 || desc->Sq == 0) return PICO_OK;
   if (!q || !out || !lse || (desc->Sk > 0 && (!k || !v)))
-    return fail(PICO_ERR_NULL, "pico_attn_fwd: q, k, v, out and lse are required");
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out))
-    return fail(PICO_ERR_ALIGN, "pico_attn_fwd: q, k, v and out must be 16-byte aligned");
+    return fail(PICO_ERR_NULL, "%s: q, k, v, out and lse are required", fn);
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(q_rot))
+    return fail(PICO_ERR_ALIGN, "%s: q, k, v, out and q_rot must be 16-byte aligned", fn);
   FwdParams p;
   p.a = make_params(desc, q, k, v);
   p.out = out;
   p.lse = lse;
   p.out_f32 = out_dtype == PICO_F32;
   p.merge = merge != 0;
+  p.rope = RopeArgs{nullptr, nullptr, 0, 0, 0, 0};
+  p.q_rot = nullptr;
+  p.qrs[0] = p.qrs[1] = p.qrs[2] = 0;
+  if (rope) {
+    if (q_pos_offset < 0) return fail(PICO_ERR_SHAPE, "%s: q_pos_offset=%d must be >= 0", fn, q_pos_offset);
+    if (int rc = check_rope_tables(fn, rope, desc->D, static_cast<int64_t>(q_pos_offset) + desc->Sq - 1)) return rc;
+    p.rope = RopeArgs{rope->cos, rope->sin, rope->pitch, rope->dtype == PICO_F32, q_pos_offset, 0};
+    if (q_rot) {
+      if (!q_rot_stride) return fail(PICO_ERR_NULL, "%s: q_rot needs its strides", fn);
+      for (int i = 0; i < 3; ++i) {
+        if (q_rot_stride[i] < 0 || q_rot_stride[i] % 8 != 0)
+          return fail(PICO_ERR_STRIDE, "%s: q_rot strides must be non-negative multiples of 8 elements", fn);
+        p.qrs[i] = q_rot_stride[i];
+      }
+      p.q_rot = static_cast<__bf16*>(q_rot);
+    }
+  }
   hipStream_t s = static_cast<hipStream_t>(stream);
   // Tile choice for D = 64: more waves per workgroup share each staged K/V tile (fewer barriers and
   // global loads per MFMA), but the launch still has to fill 256 CUs, so small problems get small tiles.
@@ -498,5 +542,19 @@ extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const vo
     else rc = launch<128, 1, 4, 64>(p, s);
   }
   if (rc) return rc;
-  return check_launch("pico_attn_fwd");
+  return check_launch(fn);
+}
+
+}  // namespace
+
+extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, void* out,
+                             float* lse, int out_dtype, int merge, void* stream) {
+  return run_fwd("pico_attn_fwd", desc, q, k, v, out, lse, out_dtype, merge, nullptr, 0, nullptr, nullptr, stream);
+}
+
+extern "C" int pico_attn_fwd_rope(const pico_attn_desc* desc, const void* q, const void* k_rot, const void* v, void* out,
+                                  float* lse, int out_dtype, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
+                                  const int64_t* q_rot_stride, void* stream) {
+  if (!rope) return fail(PICO_ERR_NULL, "pico_attn_fwd_rope: the tables are required");
+  return run_fwd("pico_attn_fwd_rope", desc, q, k_rot, v, out, lse, out_dtype, 0, rope, q_pos_offset, q_rot, q_rot_stride, stream);
 }

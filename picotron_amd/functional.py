@@ -143,31 +143,50 @@ class FusedLinearFunc(torch.autograd.Function):
         return (dx, None) + tuple(dw.split(ctx.sizes, dim=0))
 
 
+def _fused_rope() -> bool:
+    """RoPE inside the attention kernels (default); PICO_FUSED_ROPE=0 keeps it a launch of its own over q and k."""
+    import os
+    return os.getenv("PICO_FUSED_ROPE", "1") != "0"
+
+
 class QKVAttentionFunc(torch.autograd.Function):
     """RoPE on the q and k parts of a fused [B,S,(Hq+2Hkv)*D] projection, then causal / dense attention (one chunk);
-    returns [B,S,Hq*D].  The backward writes dq, dk, dv straight into the matching columns of one [B,S,(Hq+2Hkv)*D]
-    buffer and un-rotates dq and dk there in place."""
+    returns [B,S,Hq*D].
+
+    Default: q is rotated inside the attention forward (every query once, in the prologue of the workgroup that owns
+    it; the kernel leaves the rotated q behind for the backward), only k -- which many workgroups read -- is rotated by a
+    launch of its own, and the backward un-rotates dq and dk in the epilogues of its kernels: one small RoPE launch per
+    layer in the forward, none in the backward.  The backward writes dq, dk, dv straight into the matching columns of
+    one [B,S,(Hq+2Hkv)*D] buffer.  With PICO_FUSED_ROPE=0 q and k are rotated by one launch (they lie side by side in
+    the projection) and dq / dk are un-rotated in place by another."""
 
     @staticmethod
     def forward(ctx, qkv, cos, sin, n_heads, n_kv_heads, head_dim, causal):
         B, S, _ = qkv.shape
         nq, nkv = n_heads * head_dim, n_kv_heads * head_dim
         v = qkv[..., nq + nkv:].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
-        # q and k lie side by side, so one launch rotates both as Hq+Hkv heads into a [B,S,Hq+Hkv,D] copy (the
-        # projection output itself stays untouched: v is used as it lies)
-        qk = qkv[..., :nq + nkv].view(B, S, n_heads + n_kv_heads, head_dim).transpose(1, 2)
-        qk = ops.rope(qk, cos, sin, 0, out=ops.empty_bshd(B, n_heads + n_kv_heads, S, head_dim, qkv.dtype, qkv.device))
-        q, k = qk[:, :n_heads], qk[:, n_heads:]
         sm_scale = 1.0 / (head_dim ** 0.5)
-        out, lse = ops.attn_fwd(q, k, v, sm_scale, causal, 0, out_dtype=qkv.dtype, bshd_out=True)
+        fused = _fused_rope()
+        if fused:
+            q_raw = qkv[..., :nq].view(B, S, n_heads, head_dim).transpose(1, 2)
+            k_raw = qkv[..., nq:nq + nkv].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
+            k = ops.rope(k_raw, cos, sin, 0, out=ops.empty_bshd(B, n_kv_heads, S, head_dim, qkv.dtype, qkv.device))
+            out, lse, q = ops.attn_fwd_rope(q_raw, k, v, cos, sin, sm_scale, causal, 0, 0, want_q_rot=True, out_dtype=qkv.dtype)
+        else:
+            # q and k lie side by side, so one launch rotates both as Hq+Hkv heads into a [B,S,Hq+Hkv,D] copy (the
+            # projection output itself stays untouched: v is used as it lies)
+            qk = qkv[..., :nq + nkv].view(B, S, n_heads + n_kv_heads, head_dim).transpose(1, 2)
+            qk = ops.rope(qk, cos, sin, 0, out=ops.empty_bshd(B, n_heads + n_kv_heads, S, head_dim, qkv.dtype, qkv.device))
+            q, k = qk[:, :n_heads], qk[:, n_heads:]
+            out, lse = ops.attn_fwd(q, k, v, sm_scale, causal, 0, out_dtype=qkv.dtype, bshd_out=True)
         ctx.save_for_backward(q, k, v, out, lse, cos, sin)
-        ctx.meta = (n_heads, n_kv_heads, head_dim, causal, sm_scale)
+        ctx.meta = (n_heads, n_kv_heads, head_dim, causal, sm_scale, fused)
         return out.transpose(1, 2).reshape(B, S, nq)
 
     @staticmethod
     def backward(ctx, dout):
         q, k, v, out, lse, cos, sin = ctx.saved_tensors
-        n_heads, n_kv_heads, head_dim, causal, sm_scale = ctx.meta
+        n_heads, n_kv_heads, head_dim, causal, sm_scale, fused = ctx.meta
         B, S = q.size(0), q.size(2)
         nq, nkv = n_heads * head_dim, n_kv_heads * head_dim
         dqkv = torch.empty(B, S, nq + 2 * nkv, dtype=q.dtype, device=q.device)
@@ -175,9 +194,12 @@ class QKVAttentionFunc(torch.autograd.Function):
         dk = dqkv[..., nq:nq + nkv].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
         dv = dqkv[..., nq + nkv:].view(B, S, n_kv_heads, head_dim).transpose(1, 2)
         do = dout.view(B, S, n_heads, head_dim).transpose(1, 2)
-        ops.attn_bwd(do, q, k, v, lse, None, sm_scale, causal, 0, dq, dk, dv, out=out)
-        dqk = dqkv[..., :nq + nkv].view(B, S, n_heads + n_kv_heads, head_dim).transpose(1, 2)
-        ops.rope(dqk, cos, sin, 0, inverse=True, out=dqk)
+        if fused:
+            ops.attn_bwd_rope(do, q, k, v, out, lse, cos, sin, sm_scale, causal, dq, dk, dv)
+        else:
+            ops.attn_bwd(do, q, k, v, lse, None, sm_scale, causal, 0, dq, dk, dv, out=out)
+            dqk = dqkv[..., :nq + nkv].view(B, S, n_heads + n_kv_heads, head_dim).transpose(1, 2)
+            ops.rope(dqk, cos, sin, 0, inverse=True, out=dqk)
         return dqkv, None, None, None, None, None, None
 
 

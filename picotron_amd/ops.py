@@ -10,7 +10,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import PICO_BF16, PICO_F32, AttnDesc, check
+from ._lib import PICO_BF16, PICO_F32, AttnDesc, RopeTables, check
 
 _DT = {torch.bfloat16: PICO_BF16, torch.float32: PICO_F32}
 
@@ -236,6 +236,63 @@ def attn_fwd(q, k, v, sm_scale: float, causal: bool, q_offset: int = 0, out: Opt
     check(_lib.lib().pico_attn_fwd(ctypes.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(out), _ptr(lse), _dt(out, "attn_fwd out"),
                                    int(merge), _stream()))
     return out, lse
+
+
+def _rope_tables(cos: torch.Tensor, sin: torch.Tensor) -> RopeTables:
+    _dev(cos, sin)
+    if cos.dtype != sin.dtype or cos.dim() != 2 or cos.shape != sin.shape or cos.stride(-1) != 1 or sin.stride(-1) != 1 \
+            or cos.stride(0) != sin.stride(0):
+        raise RuntimeError("rope tables: cos and sin must be [positions, columns] of one dtype and row pitch, with contiguous rows")
+    t = RopeTables()
+    t.cos, t.sin, t.pitch, t.dtype, t.rows = cos.data_ptr(), sin.data_ptr(), cos.stride(0), _dt(cos, "rope tables"), cos.size(0)
+    return t
+
+
+def attn_fwd_rope(q, k_rot, v, cos, sin, sm_scale: float, causal: bool, q_offset: int = 0, q_pos_offset: int = 0,
+                  want_q_rot: bool = True, out_dtype=torch.bfloat16, bshd_out: bool = True):
+    """RoPE on q inside the attention forward (k_rot must be rotated already): returns (out, lse, q_rot or None); q_rot is
+    the rotated q, laid out like q, for attn_bwd_rope.  One chunk, no merge."""
+    _dev(q, k_rot, v)
+    q, k_rot, v = _attn_in(q, "q"), _attn_in(k_rot, "k"), _attn_in(v, "v")
+    B, Hq, Sq, D = q.shape
+    if k_rot.shape != v.shape or k_rot.size(0) != B or k_rot.size(3) != D:
+        raise RuntimeError(f"attention: shape mismatch q{tuple(q.shape)} k{tuple(k_rot.shape)} v{tuple(v.shape)}")
+    out = empty_bshd(B, Hq, Sq, D, out_dtype, q.device) if bshd_out else torch.empty(B, Hq, Sq, D, dtype=out_dtype, device=q.device)
+    lse = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+    q_rot = None
+    qrs = None
+    if want_q_rot:
+        q_rot = empty_bshd(B, Hq, Sq, D, q.dtype, q.device)
+        qrs = (ctypes.c_int64 * 3)(*q_rot.stride()[:3])
+    tables = _rope_tables(cos, sin)
+    d = _desc(q, k_rot, v, out, sm_scale, causal, q_offset)
+    check(_lib.lib().pico_attn_fwd_rope(ctypes.byref(d), _ptr(q), _ptr(k_rot), _ptr(v), _ptr(out), _ptr(lse), _dt(out, "attn out"),
+                                        ctypes.byref(tables), int(q_pos_offset), _ptr(q_rot), qrs, _stream()))
+    return out, lse, q_rot
+
+
+def attn_bwd_rope(dout, q_rot, k_rot, v, out, lse, cos, sin, sm_scale: float, causal: bool, dq, dk, dv, q_offset: int = 0,
+                  q_pos_offset: int = 0, k_pos_offset: int = 0):
+    """Backward of "rotate q and k, attend" for one chunk: writes dq / dk (gradients of the UN-rotated q and k: RoPE's
+    backward runs in the kernels' epilogues) and dv into the given buffers (any strides with a unit D stride)."""
+    _dev(dout, q_rot, k_rot, v, out, lse, dq, dk, dv)
+    q_rot, k_rot, v, dout = _attn_in(q_rot, "q"), _attn_in(k_rot, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
+    if out.stride() != dout.stride():
+        out = _like_strided(out, dout)
+    if out.dtype != torch.bfloat16:
+        raise RuntimeError("attn_bwd_rope: out must be the bf16 forward output")
+    B, Hq, Sq, D = q_rot.shape
+    if dk.dtype != dv.dtype or dk.stride() != dv.stride() or dk.stride(-1) != 1 or dq.stride(-1) != 1:
+        raise RuntimeError("attn_bwd_rope: dk and dv must share dtype and strides; dq, dk, dv need a unit D stride")
+    delta = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q_rot.device)
+    tables = _rope_tables(cos, sin)
+    d = _desc(q_rot, k_rot, v, dout, sm_scale, causal, q_offset)
+    dqs = (ctypes.c_int64 * 3)(*dq.stride()[:3])
+    dks = (ctypes.c_int64 * 3)(*dk.stride()[:3])
+    check(_lib.lib().pico_attn_bwd_rope(ctypes.byref(d), _ptr(q_rot), _ptr(k_rot), _ptr(v), _ptr(dout), _ptr(out),
+                                        _ptr(lse.contiguous()), _ptr(delta), _ptr(dq), dqs, _dt(dq, "dq"), _ptr(dk), _ptr(dv), dks,
+                                        _dt(dk, "dk/dv"), ctypes.byref(tables), int(q_pos_offset), int(k_pos_offset), _stream()))
+    return dq, dk, dv
 
 
 def attn_bwd_preprocess(dout: torch.Tensor, out: torch.Tensor, dq_acc: Optional[torch.Tensor] = None,

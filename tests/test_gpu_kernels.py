@@ -694,3 +694,57 @@ def test_empty_inputs_are_no_ops(ops, device):
     ops.adamw_lp_(e, e, e.clone(), e.clone(), 1, 1e-3)
     ops.adamw_multi_([e], [e], [e.clone()], [e.clone()], 1, 1e-3)
     torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------------------------ RoPE inside attention
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,q_offset,pos0", [
+    (2, 4, 4, 256, 256, 64, 0, 0),        # MHA, one chunk, positions from 0
+    (1, 8, 2, 200, 200, 64, 0, 37),       # GQA, ragged length, positions from 37
+    (1, 4, 2, 192, 192, 128, 0, 5),       # head_dim 128
+    (1, 4, 4, 128, 384, 64, 256, 1024),   # a query chunk behind two earlier key chunks (offset diagonal)
+    (2, 2, 1, 33, 97, 128, 64, 0),        # odd sizes
+])
+@pytest.mark.parametrize("table_dtype", [torch.bfloat16, torch.float32])
+def test_attention_with_rope_inside_vs_oracle(ops, device, B, Hq, Hkv, Sq, Sk, D, q_offset, pos0, table_dtype):
+    """pico_attn_fwd_rope / pico_attn_bwd_rope: q rotated in the forward's prologue, dq / dk un-rotated in the backward's
+    epilogues, k rotated by pico_rope -- against the oracle's apply_rotary_pos_emb + attention differentiated by
+    autograd in fp32.  Positions: key j sits at pos0 + j, query i at pos0 + q_offset + i."""
+    from oracle import layers as OL
+    from oracle import ring as OR
+    g = torch.Generator().manual_seed(100 + Sq + D)
+    q = torch.randn(B, Hq, Sq, D, generator=g).to(torch.bfloat16)
+    k = torch.randn(B, Hkv, Sk, D, generator=g).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, Sk, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, Hq, Sq, D, generator=g).to(torch.bfloat16)
+    scale = 1 / math.sqrt(D)
+    cos, sin = OL.get_cos_sin(pos0 + Sk + 3, D, 10000.0, table_dtype)
+    # oracle, fp32, on the same bf16 inputs and the same (possibly bf16-rounded) tables
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    cq, sq_ = cos[pos0 + q_offset:pos0 + q_offset + Sq].float(), sin[pos0 + q_offset:pos0 + q_offset + Sq].float()
+    ck, sk_ = cos[pos0:pos0 + Sk].float(), sin[pos0:pos0 + Sk].float()
+    q_r = OL.apply_rotary_pos_emb(qf, cq, sq_)
+    k_r = OL.apply_rotary_pos_emb(kf, ck, sk_)
+    # the reference hands bf16 tensors from the rotation to the attention (model.py:136-137): round the rotated
+    # operands the same way, with the gradient passed straight through the rounding
+    q_r = q_r + (q_r.detach().to(torch.bfloat16).float() - q_r.detach())
+    k_r = k_r + (k_r.detach().to(torch.bfloat16).float() - k_r.detach())
+    rep = Hq // Hkv
+    w_o, w_l = OR.full_attention_closed_form(q_r, k_r.repeat_interleave(rep, 1), vf.repeat_interleave(rep, 1), scale, True, q_offset)
+    gq, gk, gv = torch.autograd.grad(w_o, (qf, kf, vf), do.float())
+
+    cd, sd = cos.to(device), sin.to(device)
+    qd, kd, vd, dod = (t.to(device) for t in (q, k, v, do))
+    k_rot = ops.rope(kd, cd, sd, pos_offset=pos0)
+    out, lse, q_rot = ops.attn_fwd_rope(qd, k_rot, vd, cd, sd, scale, True, q_offset, q_pos_offset=pos0 + q_offset)
+    assert maxabs(q_rot, q_r.detach()) <= 3e-2
+    assert torch.allclose(q_rot.float(), ops.rope(qd, cd, sd, pos_offset=pos0 + q_offset).float(), rtol=2 ** -7, atol=1e-3)
+    assert maxabs(out, w_o.detach()) <= 2e-2 and maxabs(lse, w_l.detach()) <= 2e-3
+    dq = torch.empty(B, Sq, Hq, D, dtype=torch.bfloat16, device=device).transpose(1, 2)
+    dk = torch.empty(B, Sk, Hkv, D, dtype=torch.bfloat16, device=device).transpose(1, 2)
+    dv = torch.empty_like(dk)
+    ops.attn_bwd_rope(dod, q_rot, k_rot, vd, out, lse, cd, sd, scale, True, dq, dk, dv, q_offset,
+                      q_pos_offset=pos0 + q_offset, k_pos_offset=pos0)
+    assert rel_l2(dq, gq) <= 1e-2 and rel_l2(dk, gk) <= 1e-2 and rel_l2(dv, gv) <= 1e-2
+    # and the same numbers as the separate-launch path, up to the rounding the fused path does not do twice
+    o2, l2 = ops.attn_fwd(q_rot, k_rot, vd, scale, True, q_offset)
+    assert torch.equal(o2, out) and torch.equal(l2, lse)

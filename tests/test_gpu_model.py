@@ -368,3 +368,31 @@ def test_chained_residual_stream_matches_separate_adds(pgm1, device):
     for n, g0 in res["0"][2].items():
         assert res["1"][2][n].dtype == g0.dtype
         assert rel_l2(res["1"][2][n], g0) <= 2e-2, n
+
+
+def test_rope_inside_attention_matches_separate_rope_launches(pgm1, device):
+    """PICO_FUSED_ROPE: q rotated inside the attention forward, dq / dk un-rotated inside the backward kernels (one
+    RoPE launch per layer, on k, instead of two on q and k) must give the loss and gradients of the path that rotates
+    q and k with launches of their own; MHA and GQA."""
+    from picotron_amd.functional import cross_entropy
+    from picotron_amd.model import Llama
+    for heads, kv in ((4, 4), (8, 2)):
+        cfg = OM.LlamaShape(64 * heads, heads, kv, 512, 1024, 2, 160)
+        ids, tgt = OM.synthetic_batch(cfg.vocab_size, 2, 160, seed=9)
+        ids, tgt = ids.to(device), tgt.to(device)
+        res = {}
+        try:
+            for mode in ("0", "1"):
+                os.environ["PICO_FUSED_ROPE"] = mode
+                torch.manual_seed(0)
+                m = Llama(cfg).to(device).to(torch.bfloat16)
+                logits = m(ids)
+                loss = cross_entropy(logits.view(-1, cfg.vocab_size), tgt.reshape(-1))
+                loss.backward()
+                res[mode] = (loss.item(), logits.detach().float().cpu(), {n: p.grad.float().cpu() for n, p in m.named_parameters()})
+        finally:
+            os.environ.pop("PICO_FUSED_ROPE", None)
+        assert abs(res["0"][0] - res["1"][0]) <= 2e-3
+        assert rel_l2(res["1"][1], res["0"][1]) <= 1e-2
+        for n, g0 in res["0"][2].items():
+            assert rel_l2(res["1"][2][n], g0) <= 2e-2, n
