@@ -98,7 +98,8 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   const int hq = blockIdx.x % a.Hq, b = blockIdx.x / a.Hq;
   const int hkv = hq / (a.Hq / a.Hkv);
   const int q0 = qtile * BM;
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);   // uniform over the wave: lets wave-dependent tests be scalar branches
   const int n = lane % 32, h = lane / 32;
   const int qw = wave % C::kQWaves, ks = wave / C::kQWaves;   // which queries, which 64-key step of a staged tile
 
