@@ -36,7 +36,8 @@ __device__ __forceinline__ u32x4 load_raw(const void* p) {
 constexpr int kFwdThreads = 256;
 constexpr int kBwdThreads = 512;
 constexpr int kMaxBwdBlocks = 512;   // rows of the dweight workspace
-constexpr int kBwdWaveThreads = 256; // block size of the row-per-wave backward
+constexpr int kBwdWaves = 4;         // waves per block of the row-per-wave backward
+
 
 template <int G>
 __device__ __forceinline__ float group_sum(float v, float* smem /* this group's 4 floats, G == 256 only */) {
@@ -206,38 +207,45 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
 // next row: loads and stores retire in one order, so waiting for a prefetched row also waits for the stores
 // of the current one (measured: 3.4 TB/s with the prefetch, 5.2 TB/s -- the rate of a plain copy -- without).  The block's four waves are summed through LDS once at
 // the end and the block writes one row of the partial-sum workspace.
-template <typename T, int NV, bool kRes>
-__global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
+template <typename T, int NV, bool kRes, int R, int NWAVE>
+__global__ __launch_bounds__(NWAVE * kWave) void rmsnorm_bwd_wave_kernel(
     const T* __restrict__ dy, const T* __restrict__ x, const T* __restrict__ w,
     const float* __restrict__ rstd, const T* dres, T* dx, float* __restrict__ partial,
     int64_t rows, int hidden) {
   constexpr int V = io<T>::kVec;
-  constexpr int NWAVE = kBwdWaveThreads / kWave;
-  extern __shared__ float red[];  // [NWAVE - 1][hidden]
-  const int wave = threadIdx.x / kWave, t = threadIdx.x % kWave;
+  extern __shared__ __attribute__((aligned(16))) float red[];  // [NWAVE][hidden]
+  const int t = threadIdx.x % kWave;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);   // uniform: row addresses become scalar base + lane offset
   const int nvec = hidden / V;
   const float inv_h = 1.f / static_cast<float>(hidden);
-  float dw[NV][V], wv[NV][V];
-  u32x4 xr[NV], dr[NV], rr[kRes ? NV : 1];  // rr: the residual stream's own gradient (kRes: dres is given)
-  float rs;
+  float dw[NV][V];
+  // The weight stays packed (16 bytes per piece) and is unpacked where it is used: unpacked it would double its
+  // registers, and registers decide how many rows the GPU has in flight (asm_keep stops the compiler from hoisting the
+  // unpacking out of the row loop).
+  u32x4 wp[NV];
+  // R rows of the wave are in flight together: all their loads are issued before the first is waited for, so a wave
+  // that owns R rows pays one memory latency for them, not R
+  u32x4 xr[R][NV], dr[R][NV], rr[R][kRes ? NV : 1];  // rr: the residual stream's own gradient (kRes: dres is given)
+  float rs[R];
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
 #pragma unroll
-    for (int e = 0; e < V; ++e) { dw[j][e] = 0.f; wv[j][e] = 0.f; }
-    if (t + j * kWave < nvec) io<T>::load(w + (t + j * kWave) * V, wv[j]);
+    for (int e = 0; e < V; ++e) dw[j][e] = 0.f;
+    const int v = t + j * kWave;
+    wp[j] = *reinterpret_cast<const u32x4*>(w + (v < nvec ? v : 0) * V);
   }
   const int64_t stride = static_cast<int64_t>(gridDim.x) * NWAVE;
   int64_t row = static_cast<int64_t>(blockIdx.x) * NWAVE + wave;
-  auto fetch = [&](int64_t r) {
+  auto fetch = [&](int q, int64_t r) {
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
       const int v = t + j * kWave;
       const int vc = v < nvec ? v : 0;
-      xr[j] = load_raw(x + r * hidden + vc * V);
-      dr[j] = load_raw(dy + r * hidden + vc * V);
-      if constexpr (kRes) rr[j] = load_raw(dres + r * hidden + vc * V);
+      xr[q][j] = load_raw(x + r * hidden + vc * V);
+      dr[q][j] = load_raw(dy + r * hidden + vc * V);
+      if constexpr (kRes) rr[q][j] = load_raw(dres + r * hidden + vc * V);
     }
-    rs = rstd[r];
+    rs[q] = rstd[r];
   };
   auto unpack = [&](const u32x4& raw, float (&out)[V]) {
     if constexpr (V == 8) {
@@ -251,71 +259,84 @@ __global__ __launch_bounds__(kBwdWaveThreads) void rmsnorm_bwd_wave_kernel(
       for (int i = 0; i < 4; ++i) out[i] = __uint_as_float(raw[i]);
     }
   };
-  for (; row < rows; row += stride) {
-    fetch(row);
-    const float r = rs;
-    float c = 0.f;
+  for (; row < rows; row += R * stride) {
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      if (t + j * kWave < nvec) {
-        float xv[V], dv[V];
-        unpack(xr[j], xv);
-        unpack(dr[j], dv);
-#pragma unroll
-        for (int e = 0; e < V; ++e) {
-          const float xh = xv[e] * r;
-          c += dv[e] * wv[j][e] * xh;
-          dw[j][e] += dv[e] * xh;
-        }
-      }
+    for (int q = 0; q < R; ++q) {
+      const int64_t rq = row + q * stride;
+      fetch(q, rq < rows ? rq : row);   // a row past the end re-reads the first one; nothing of it is used
     }
-    c = wave_sum(c) * inv_h;
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int v = t + j * kWave;
-      if (v < nvec) {
-        float xv[V], dv[V], o[V];
-        unpack(xr[j], xv);
-        unpack(dr[j], dv);
+    for (int j = 0; j < NV; ++j) asm volatile("" : "+v"(wp[j]));
 #pragma unroll
-        for (int e = 0; e < V; ++e) o[e] = r * (dv[e] * wv[j][e] - xv[e] * r * c);
-        if constexpr (kRes) {  // dx may alias dres: this lane read its part of the row before it writes it
-          float rv[V];
-          unpack(rr[j], rv);
+    for (int q = 0; q < R; ++q) {
+      const int64_t rq = row + q * stride;
+      if (rq >= rows) break;
+      const float r = rs[q];
+      float c = 0.f;
 #pragma unroll
-          for (int e = 0; e < V; ++e) o[e] += rv[e];
+      for (int j = 0; j < NV; ++j) {
+        if (t + j * kWave < nvec) {
+          float xv[V], dv[V], wv[V];
+          unpack(xr[q][j], xv);
+          unpack(dr[q][j], dv);
+          unpack(wp[j], wv);
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            const float xh = xv[e] * r;
+            c += dv[e] * wv[e] * xh;
+            dw[j][e] += dv[e] * xh;
+          }
         }
-        store_as<T, PICO_NT_NORM_BWD != 0>(dx + row * hidden + v * V, o);
+        __builtin_amdgcn_sched_barrier(0);   // one piece at a time: pieces unpacked side by side cost registers
+      }
+      c = wave_sum(c) * inv_h;
+      // the second pass unpacks the row again: keeping the first pass's products alive for it would cost 2 x the
+      // row's share in registers (the empty asm hides from the compiler that the values are the same)
+#pragma unroll
+      for (int j = 0; j < NV; ++j) asm volatile("" : "+v"(xr[q][j]), "+v"(dr[q][j]), "+v"(wp[j]));
+#pragma unroll
+      for (int j = 0; j < NV; ++j) {
+        const int v = t + j * kWave;
+        if (v < nvec) {
+          float xv[V], dv[V], wv[V], o[V];
+          unpack(xr[q][j], xv);
+          unpack(dr[q][j], dv);
+          unpack(wp[j], wv);
+#pragma unroll
+          for (int e = 0; e < V; ++e) o[e] = r * (dv[e] * wv[e] - xv[e] * r * c);
+          if constexpr (kRes) {  // dx may alias dres: this lane read its part of the row before it writes it
+            float rv[V];
+            unpack(rr[q][j], rv);
+#pragma unroll
+            for (int e = 0; e < V; ++e) o[e] += rv[e];
+          }
+          store_as<T, PICO_NT_NORM_BWD != 0>(dx + rq * hidden + v * V, o);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
   }
-  // block reduction of dweight: waves 1.. park their share in LDS, wave 0 adds and writes the partial row
-  if (wave > 0) {
+  // block reduction of dweight: every wave parks its share in LDS, then all threads sum columns (a fixed order) and
+  // write the block's row of the partial sums
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int v = t + j * kWave;
-      if (v < nvec) {
-#pragma unroll
-        for (int e = 0; e < V; ++e) red[(wave - 1) * hidden + v * V + e] = dw[j][e];
+  for (int j = 0; j < NV; ++j) {
+    const int v = t + j * kWave;
+    if (v < nvec) {
+      if constexpr (V == 8) {
+        *reinterpret_cast<f32x4*>(&red[wave * hidden + v * V]) = f32x4{dw[j][0], dw[j][1], dw[j][2], dw[j][3]};
+        *reinterpret_cast<f32x4*>(&red[wave * hidden + v * V + 4]) = f32x4{dw[j][4], dw[j][5], dw[j][6], dw[j][7]};
+      } else {
+        *reinterpret_cast<f32x4*>(&red[wave * hidden + v * V]) = f32x4{dw[j][0], dw[j][1], dw[j][2], dw[j][3]};
       }
     }
   }
   __syncthreads();
-  if (wave == 0) {
-    float* out = partial + static_cast<int64_t>(blockIdx.x) * hidden;
+  float* out = partial + static_cast<int64_t>(blockIdx.x) * hidden;
+  for (int c4 = threadIdx.x * 4; c4 < hidden; c4 += NWAVE * kWave * 4) {
+    f32x4 acc = *reinterpret_cast<const f32x4*>(&red[c4]);
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int v = t + j * kWave;
-      if (v < nvec) {
-#pragma unroll
-        for (int e = 0; e < V; ++e) {
-          float acc = dw[j][e];
-#pragma unroll
-          for (int k = 0; k < NWAVE - 1; ++k) acc += red[k * hidden + v * V + e];
-          out[v * V + e] = acc;
-        }
-      }
-    }
+    for (int k = 1; k < NWAVE; ++k) acc += *reinterpret_cast<const f32x4*>(&red[k * hidden + c4]);
+    *reinterpret_cast<f32x4*>(&out[c4]) = acc;
   }
 }
 
@@ -445,20 +466,23 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
   }
 #define PICO_BWD_WAVE(NV)                                                                              \
   {                                                                                                    \
-    const int blocks = bwd_blocks(rows, kBwdWaveThreads / kWave, hidden);                                      \
+    const int blocks = bwd_blocks(rows, kBwdWaves, hidden);                                            \
     *blocks_out = blocks;                                                                              \
-    const size_t lds = static_cast<size_t>(kBwdWaveThreads / kWave - 1) * hidden * sizeof(float);      \
-    if (dres)                                                                                          \
-      hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV, true>), dim3(blocks), dim3(kBwdWaveThreads), lds, s, \
+    const size_t lds = static_cast<size_t>(kBwdWaves) * hidden * sizeof(float);                        \
+    auto go = [&](auto kern, std::atomic<bool>& reserved) -> int {                                     \
+      if (lds > 48 * 1024 && !reserve_lds_once(reserved, reinterpret_cast<const void*>(kern),          \
+                                               kBwdWaves * 64 * NV * io<T>::kVec * sizeof(float)))     \
+        return fail(PICO_ERR_LAUNCH, "pico_rmsnorm_bwd: cannot reserve %zu bytes of LDS", lds);        \
+      hipLaunchKernelGGL(kern, dim3(blocks), dim3(kBwdWaves * kWave), lds, s,                          \
                          static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), \
                          rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
-    else                                                                                               \
-      hipLaunchKernelGGL((rmsnorm_bwd_wave_kernel<T, NV, false>), dim3(blocks), dim3(kBwdWaveThreads), lds, s, \
-                         static_cast<const T*>(dy), static_cast<const T*>(x), static_cast<const T*>(w), \
-                         rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
-    return PICO_OK;                                                                                    \
+      return PICO_OK;                                                                                  \
+    };                                                                                                 \
+    static std::atomic<bool> reserved_res{false}, reserved_plain{false};                               \
+    if (dres) return go(rmsnorm_bwd_wave_kernel<T, NV, true, 1, kBwdWaves>, reserved_res);             \
+    return go(rmsnorm_bwd_wave_kernel<T, NV, false, 1, kBwdWaves>, reserved_plain);                    \
   }
-  if (nv_wave) {   // rows of at most 64 x 8 vectors: (4 - 1) waves x hidden floats of LDS is at most 48 KiB
+  if (nv_wave) {   // rows of at most 64 x 8 vectors: 4 waves x hidden floats of LDS is at most 64 KiB
     switch (nv_wave) {
       case 1: PICO_BWD_WAVE(1);
       case 2: PICO_BWD_WAVE(2);
@@ -485,10 +509,8 @@ int64_t bwd_partial_bytes(int64_t rows, int64_t hidden, int dtype) {
   const int vec = dtype == PICO_BF16 ? 8 : 4;
   const int nvec = static_cast<int>(hidden / vec);
   const int nv_wave = pick_nv((nvec + 63) / 64, 8);
-  int gpb;
-  if (nv_wave) gpb = kBwdWaveThreads / kWave;
-  else gpb = kBwdThreads / 256;
-  return static_cast<int64_t>(bwd_blocks(rows, gpb, static_cast<int>(hidden))) * hidden * static_cast<int64_t>(sizeof(float));
+  if (nv_wave) return static_cast<int64_t>(bwd_blocks(rows, kBwdWaves, static_cast<int>(hidden))) * hidden * static_cast<int64_t>(sizeof(float));
+  return static_cast<int64_t>(bwd_blocks(rows, kBwdThreads / 256, static_cast<int>(hidden))) * hidden * static_cast<int64_t>(sizeof(float));
 }
 
 int check_common(const char* fn, int64_t rows, int64_t hidden, int dtype) {
