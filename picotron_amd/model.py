@@ -78,13 +78,37 @@ class TritonRMSNorm(nn.Module):
 
     def forward(self, hidden_states, residual=None, dropout_p=0.0, prenorm=False, residual_in_fp32=False,
                 return_dropout_mask=False):
-        if dropout_p != 0.0 or return_dropout_mask or residual_in_fp32:
-            raise NotImplementedError("TritonRMSNorm: dropout and fp32 residuals are not used by picotron and not built")
-        if residual is None:
-            y = RMSNormFunc.apply(hidden_states, self.weight, self.eps, False)
-            return (y, hidden_states) if prenorm else y
-        y, h = RMSNormResidualFunc.apply(hidden_states, residual, self.weight, self.eps)
-        return (y, h) if prenorm else y
+        """The call shape of flash-attn's ``layer_norm_fn(..., is_rms_norm=True)`` as the reference passes it through
+        (``model.py:54-65``): h = dropout(x) + residual, y = rmsnorm(h) * w in x's dtype; ``prenorm`` also returns h
+        (in fp32 if ``residual_in_fp32``), ``return_dropout_mask`` appends the keep mask and a None (the second
+        input's mask, which does not exist here).  picotron itself calls it without dropout and with residuals in the
+        activations' dtype: those calls take the fused kernels; dropout and the fp32 add are torch operations in front
+        of the norm kernel."""
+        if dropout_p == 0.0 and not return_dropout_mask and not residual_in_fp32:
+            if residual is None:
+                y = RMSNormFunc.apply(hidden_states, self.weight, self.eps, False)
+                return (y, hidden_states) if prenorm else y
+            y, h = RMSNormResidualFunc.apply(hidden_states, residual, self.weight, self.eps)
+            return (y, h) if prenorm else y
+        x = hidden_states
+        mask = None
+        h = x.float()
+        if dropout_p > 0.0:
+            mask = torch.rand_like(h) >= dropout_p
+            h = h * mask * (1.0 / (1.0 - dropout_p))
+        elif return_dropout_mask:
+            mask = torch.ones_like(h, dtype=torch.bool)
+        if residual is not None:
+            h = h + residual.float()
+        if residual_in_fp32:
+            y = RMSNormFunc.apply(h, self.weight.float(), self.eps, False).to(x.dtype)
+        else:
+            h = h.to(x.dtype if residual is None else residual.dtype)
+            y = RMSNormFunc.apply(h.to(x.dtype), self.weight, self.eps, False)
+        out = (y, h) if prenorm else (y,)
+        if return_dropout_mask:
+            out = out + (mask, None)
+        return out if len(out) > 1 else out[0]
 
 
 class LlamaRMSNorm(nn.Module):

@@ -124,8 +124,22 @@ def test_norm_modules_with_the_reference_argument_lists(device, dtype):
     want_sum = (x.float() + res.float()).to(dtype)
     assert maxabs(hsum, want_sum.float()) <= (4e-2 if dtype == torch.bfloat16 else 1e-6)
     assert maxabs(y, OL.rmsnorm(hsum.float().cpu(), w.float(), eps, cast_then_scale=False)) <= tol
-    with pytest.raises(NotImplementedError):
-        triton(x.to(device), dropout_p=0.1)
+    # dropout_p / residual_in_fp32 / return_dropout_mask, the rest of layer_norm_fn's argument list: the returned keep
+    # mask fixes the expected value (h = x * mask / (1 - p) + residual, kept in fp32 when asked; y = rmsnorm(h) * w)
+    torch.manual_seed(11)
+    y, hsum, mask, mask1 = triton(x.to(device), residual=res.to(device), dropout_p=0.25, prenorm=True, residual_in_fp32=True,
+                                  return_dropout_mask=True)
+    assert mask1 is None and mask.dtype == torch.bool and 0.6 < mask.float().mean().item() < 0.9
+    want_h = x.float() * mask.cpu() / 0.75 + res.float()
+    assert hsum.dtype == torch.float32 and maxabs(hsum, want_h) <= 1e-5
+    assert y.dtype == dtype and maxabs(y, OL.rmsnorm(want_h, w.float(), eps, cast_then_scale=False)) <= tol
+    y2, mask2, _ = triton(x.to(device), dropout_p=0.0, return_dropout_mask=True)
+    assert bool(mask2.all()) and maxabs(y2, OL.rmsnorm(x.float(), w.float(), eps, cast_then_scale=False)) <= tol
+    # and gradients flow through the composed path
+    xg = x.to(device).requires_grad_()
+    y3, h3 = triton(xg, residual=res.to(device), prenorm=True, residual_in_fp32=True)
+    (y3.float().sum() + h3.sum()).backward()
+    assert xg.grad is not None and triton.weight.grad is not None and torch.isfinite(xg.grad.float()).all()
 
 
 def test_mlp_module_matches_the_oracle_formula(device):
