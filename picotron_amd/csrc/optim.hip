@@ -13,52 +13,20 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kPerThread = 8;  // elements: one 16-byte bf16 vector, two 16-byte fp32 vectors per state
 
-// streaming switches: the optimizer touches every byte once per step and its working set is far larger than any cache.
-// Loads and stores together: +16 % with all-bf16 state; either alone changes nothing or costs 3 %.
-#ifndef PICO_NT_ADAMW_LOADS
-#define PICO_NT_ADAMW_LOADS 1
-#endif
-#ifndef PICO_NT_ADAMW_STORES
-#define PICO_NT_ADAMW_STORES 1
-#endif
-#ifndef PICO_ADAMW_SPLIT
-#define PICO_ADAMW_SPLIT 1
-#endif
 __device__ __forceinline__ void load8(const float* p, float (&out)[8]) {
-  float a[4], b[4];
-  load_as<float, PICO_NT_ADAMW_LOADS != 0>(p, a);
-  load_as<float, PICO_NT_ADAMW_LOADS != 0>(p + 4, b);
+  const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
 #pragma unroll
   for (int i = 0; i < 4; ++i) { out[i] = a[i]; out[4 + i] = b[i]; }
 }
 __device__ __forceinline__ void store8(float* p, const float (&in)[8]) {
-  float a[4], b[4];
+  f32x4 a, b;
 #pragma unroll
   for (int i = 0; i < 4; ++i) { a[i] = in[i]; b[i] = in[4 + i]; }
-  store_as<float, PICO_NT_ADAMW_STORES != 0>(p, a);
-  store_as<float, PICO_NT_ADAMW_STORES != 0>(p + 4, b);
+  *reinterpret_cast<f32x4*>(p) = a;
+  *reinterpret_cast<f32x4*>(p + 4) = b;
 }
-__device__ __forceinline__ void load8(const __bf16* p, float (&out)[8]) { load_as<__bf16, PICO_NT_ADAMW_LOADS != 0>(p, out); }
-__device__ __forceinline__ void store8(__bf16* p, const float (&in)[8]) { store_as<__bf16, PICO_NT_ADAMW_STORES != 0>(p, in); }
-// four consecutive elements: 16 bytes of fp32, 8 bytes of bf16
-__device__ __forceinline__ void load4(const float* p, float (&out)[4]) { load_as<float, PICO_NT_ADAMW_LOADS != 0>(p, out); }
-__device__ __forceinline__ void store4(float* p, const float (&in)[4]) { store_as<float, PICO_NT_ADAMW_STORES != 0>(p, in); }
-__device__ __forceinline__ void load4(const __bf16* p, float (&out)[4]) {
-#if PICO_NT_ADAMW_LOADS
-  const u32x2 raw = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
-#else
-  const u32x2 raw = *reinterpret_cast<const u32x2*>(p);
-#endif
-  out[0] = __uint_as_float(raw[0] << 16);  out[1] = __uint_as_float(raw[0] & 0xffff0000u);
-  out[2] = __uint_as_float(raw[1] << 16);  out[3] = __uint_as_float(raw[1] & 0xffff0000u);
-}
-__device__ __forceinline__ void store4(__bf16* p, const float (&in)[4], bool stream) {
-  u32x2 raw;
-  raw[0] = pack_bf16x2(in[0], in[1]);
-  raw[1] = pack_bf16x2(in[2], in[3]);
-  if (stream && PICO_NT_ADAMW_STORES != 0) __builtin_nontemporal_store(raw, reinterpret_cast<u32x2*>(p));
-  else *reinterpret_cast<u32x2*>(p) = raw;
-}
+__device__ __forceinline__ void load8(const __bf16* p, float (&out)[8]) { io<__bf16>::load(p, out); }
+__device__ __forceinline__ void store8(__bf16* p, const float (&in)[8]) { io<__bf16>::store(p, in); }
 
 // The arithmetic follows torch.optim.AdamW's (non-amsgrad) order of operations so that fp32 states match it to
 // rounding: p *= 1 - lr*wd;  m = m + (g - m)*(1 - b1);  v = v*b2 + g*g*(1 - b2);
@@ -103,7 +71,7 @@ __device__ __forceinline__ void adamw_block(__bf16* __restrict__ param_lp, TW* _
     store8(master + i0, p);
     store8(exp_avg + i0, m);
     store8(exp_avg_sq + i0, v);
-    if (param_lp) io<__bf16>::store(param_lp + i0, p);   // the model reads this copy next: a normal store
+    if (param_lp) io<__bf16>::store(param_lp + i0, p);
   } else {
     for (int e = 0; e < kPerThread && i0 + e < n; ++e) {
       master[i0 + e] = static_cast<TW>(p[e]);
@@ -114,81 +82,11 @@ __device__ __forceinline__ void adamw_block(__bf16* __restrict__ param_lp, TW* _
   }
 }
 
-// The same step with another element-to-lane map, for fp32 moments: a lane takes two groups of four consecutive
-// elements, 256 elements apart within its wave's 512, so that every fp32 access of a wave is 1 KiB of consecutive
-// bytes (the map above gives a lane 32 consecutive bytes of an fp32 array: two instructions that each touch every
-// other 16 bytes of 2 KiB); bf16 arrays are then read 8 bytes per lane.
-template <typename TW, typename TM, typename TG>
-__device__ __forceinline__ void adamw_block_split(__bf16* __restrict__ param_lp, TW* __restrict__ master,
-                                                  const TG* __restrict__ grad, TM* __restrict__ exp_avg,
-                                                  TM* __restrict__ exp_avg_sq, int64_t n, int64_t block, const Hyper& h) {
-  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int64_t base = (block * (kThreads / kWave) + wave) * (kWave * kPerThread);
-  if (base >= n) return;
-  if (base + kWave * kPerThread > n) {   // the tensor's last, partial piece: element by element
-    for (int e = 0; e < kPerThread; ++e) {
-      const int64_t i = base + (e / 4) * (kWave * 4) + lane * 4 + (e % 4);
-      if (i < n) {
-        const float ge = static_cast<float>(grad[i]) * h.grad_scale;
-        float pe = static_cast<float>(master[i]) * h.decay;
-        float me = static_cast<float>(exp_avg[i]), ve = static_cast<float>(exp_avg_sq[i]);
-        me = me + (ge - me) * h.one_minus_b1;
-        ve = ve * h.b2 + ge * ge * h.one_minus_b2;
-        pe = pe - h.step_size * (me / (__builtin_sqrtf(ve) * h.inv_sqrt_bc2 + h.eps));
-        master[i] = static_cast<TW>(pe);
-        exp_avg[i] = static_cast<TM>(me);
-        exp_avg_sq[i] = static_cast<TM>(ve);
-        if (param_lp) param_lp[i] = static_cast<__bf16>(pe);
-      }
-    }
-    return;
-  }
-  float g[2][4], p[2][4], m[2][4], v[2][4];
-#pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int64_t i = base + q * (kWave * 4) + lane * 4;
-    load4(grad + i, g[q]);
-    load4(master + i, p[q]);
-    load4(exp_avg + i, m[q]);
-    load4(exp_avg_sq + i, v[q]);
-  }
-#pragma unroll
-  for (int q = 0; q < 2; ++q)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float ge = g[q][e] * h.grad_scale;
-      p[q][e] = p[q][e] * h.decay;
-      m[q][e] = m[q][e] + (ge - m[q][e]) * h.one_minus_b1;
-      v[q][e] = v[q][e] * h.b2 + ge * ge * h.one_minus_b2;
-      const float denom = __builtin_sqrtf(v[q][e]) * h.inv_sqrt_bc2 + h.eps;
-      p[q][e] = p[q][e] - h.step_size * (m[q][e] / denom);
-    }
-#pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int64_t i = base + q * (kWave * 4) + lane * 4;
-    if constexpr (sizeof(TW) == 4) store4(master + i, p[q]);
-    else store4(master + i, p[q], false);   // the model reads the updated bf16 parameter next: a normal store
-    store4(exp_avg + i, m[q]);
-    store4(exp_avg_sq + i, v[q]);
-    if (param_lp) store4(param_lp + i, p[q], false);
-  }
-}
-
-template <typename TW, typename TM, typename TG>
-__device__ __forceinline__ void adamw_step(__bf16* __restrict__ param_lp, TW* __restrict__ master,
-                                           const TG* __restrict__ grad, TM* __restrict__ exp_avg,
-                                           TM* __restrict__ exp_avg_sq, int64_t n, int64_t block, const Hyper& h) {
-  if constexpr (PICO_ADAMW_SPLIT != 0 && sizeof(TM) == 4)
-    adamw_block_split<TW, TM, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, block, h);
-  else
-    adamw_block<TW, TM, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, block, h);
-}
-
 template <typename TW, typename TM, typename TG>
 __global__ __launch_bounds__(kThreads) void adamw_kernel(__bf16* __restrict__ param_lp, TW* __restrict__ master,
                                                          const TG* __restrict__ grad, TM* __restrict__ exp_avg,
                                                          TM* __restrict__ exp_avg_sq, int64_t n, Hyper h) {
-  adamw_step<TW, TM, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, blockIdx.x, h);
+  adamw_block<TW, TM, TG>(param_lp, master, grad, exp_avg, exp_avg_sq, n, blockIdx.x, h);
 }
 
 // Many tensors in one launch: the pointers travel in the kernel arguments (no table in device memory to keep alive),
@@ -213,7 +111,7 @@ __global__ __launch_bounds__(kThreads) void adamw_multi_kernel(TensorTable t, Hy
     const int mid = (lo + hi) >> 1;
     if (bid >= t.block_start[mid]) lo = mid; else hi = mid;
   }
-  adamw_step<TW, TM, TG>(static_cast<__bf16*>(t.param_lp[lo]), static_cast<TW*>(t.weight[lo]),
+  adamw_block<TW, TM, TG>(static_cast<__bf16*>(t.param_lp[lo]), static_cast<TW*>(t.weight[lo]),
                           static_cast<const TG*>(t.grad[lo]), static_cast<TM*>(t.exp_avg[lo]),
                           static_cast<TM*>(t.exp_avg_sq[lo]), t.n[lo], bid - t.block_start[lo], h);
 }
