@@ -84,6 +84,56 @@ def test_seeded_shape_sweep(device):
     assert not failures, failures
 
 
+def test_seeded_sweep_of_rope_inside_attention(device):
+    """pico_attn_fwd_rope / pico_attn_bwd_rope over 40 seeded shapes (every launch-size class, GQA, ragged lengths,
+    position offsets, both table dtypes) against the same kernels fed by separate RoPE launches: identical forward
+    (the rotated q is bit-equal), gradients equal up to the one rounding the fused path does not do twice."""
+    from picotron_amd import ops
+    from oracle import layers as OL
+    failures = []
+    for case, B, Hq, Hkv, Sq, Sk, D, causal, q_offset in cases(40, seed=77):
+        rng = random.Random(case)
+        pos0 = rng.choice([0, 0, 3, 129, 1000])
+        tdt = rng.choice([torch.bfloat16, torch.float32])
+        g = torch.Generator().manual_seed(500 + case)
+        q = torch.randn(B, Sq, Hq, D, generator=g).to(torch.bfloat16).to(device).transpose(1, 2)
+        k = torch.randn(B, Sk, Hkv, D, generator=g).to(torch.bfloat16).to(device).transpose(1, 2)
+        v = torch.randn(B, Sk, Hkv, D, generator=g).to(torch.bfloat16).to(device).transpose(1, 2)
+        do = torch.randn(B, Sq, Hq, D, generator=g).to(torch.bfloat16).to(device).transpose(1, 2)
+        scale = 1 / math.sqrt(D)
+        cos, sin = OL.get_cos_sin(pos0 + q_offset + max(Sq, Sk) + 1, D, 10000.0, tdt)
+        cos, sin = cos.to(device), sin.to(device)
+        qp, kp = pos0 + q_offset, pos0
+        k_rot = ops.rope(k, cos, sin, pos_offset=kp)
+        q_rot_ref = ops.rope(q, cos, sin, pos_offset=qp)
+        o0, l0 = ops.attn_fwd(q_rot_ref, k_rot, v, scale, causal, q_offset, bshd_out=True)
+        o1, l1, q_rot = ops.attn_fwd_rope(q, k_rot, v, cos, sin, scale, causal, q_offset, q_pos_offset=qp)
+        bad = []
+        if not (torch.equal(q_rot, q_rot_ref) and torch.equal(o0, o1) and torch.equal(l0, l1)):
+            bad.append("forward")
+
+        def grads():
+            return (torch.empty(B, Sq, Hq, D, dtype=torch.bfloat16, device=device).transpose(1, 2),
+                    torch.empty(B, Sk, Hkv, D, dtype=torch.bfloat16, device=device).transpose(1, 2),
+                    torch.empty(B, Sk, Hkv, D, dtype=torch.bfloat16, device=device).transpose(1, 2))
+        dq0, dk0, dv0 = grads()
+        ops.attn_bwd(do, q_rot, k_rot, v, l0, None, scale, causal, q_offset, dq0, dk0, dv0, out=o0)
+        dq0 = ops.rope(dq0, cos, sin, pos_offset=qp, inverse=True)
+        dk0 = ops.rope(dk0, cos, sin, pos_offset=kp, inverse=True)
+        dq1, dk1, dv1 = grads()
+        ops.attn_bwd_rope(do, q_rot, k_rot, v, o1, l1, cos, sin, scale, causal, dq1, dk1, dv1, q_offset,
+                          q_pos_offset=qp, k_pos_offset=kp)
+        if not torch.equal(dv0, dv1):
+            bad.append("dv")
+        if rel_l2(dq1, dq0) > 6e-3:
+            bad.append("dq")
+        if rel_l2(dk1, dk0) > 6e-3:
+            bad.append("dk")
+        if bad:
+            failures.append((case, B, Hq, Hkv, Sq, Sk, D, causal, q_offset, pos0, str(tdt), bad))
+    assert not failures, failures
+
+
 def test_seeded_sweep_of_the_bandwidth_kernels(device):
     """RMSNorm (both rounding orders, with and without the fused residual), SwiGLU and cross-entropy, forward and
     backward, at 40 seeded sizes against torch in fp32 on the GPU."""
