@@ -18,6 +18,12 @@ constexpr int kWaves = kThreads / kWave;
 #ifndef PICO_NT_CE_BWD_LOADS
 #define PICO_NT_CE_BWD_LOADS 1
 #endif
+#ifndef PICO_CE_BWD_UNROLL
+#define PICO_CE_BWD_UNROLL 4
+#endif
+#ifndef PICO_CE_FWD_UNROLL
+#define PICO_CE_FWD_UNROLL 2
+#endif
 #ifndef PICO_NT_CE_BWD_STORES
 #define PICO_NT_CE_BWD_STORES 1
 #endif
@@ -39,9 +45,7 @@ __global__ __launch_bounds__(kThreads) void ce_fwd_kernel(const T* __restrict__ 
   const int nvec = vocab / V;
   // online (max, sum of exp) per thread, in the log2 domain
   float m = -INFINITY, s = 0.f;
-  for (int v = threadIdx.x; v < nvec; v += kThreads) {
-    float e[V];
-    load_as<T, PICO_NT_CE_FWD_LOADS != 0>(x + static_cast<int64_t>(v) * V, e);
+  auto absorb = [&](const float (&e)[V]) {
     float mx = e[0];
 #pragma unroll
     for (int i = 1; i < V; ++i) mx = fmaxf(mx, e[i]);
@@ -49,6 +53,20 @@ __global__ __launch_bounds__(kThreads) void ce_fwd_kernel(const T* __restrict__ 
     if (mx > m) { s *= fast_exp2(m - mx); m = mx; }
 #pragma unroll
     for (int i = 0; i < V; ++i) s += fast_exp2(e[i] * kLog2e - m);
+  };
+  constexpr int U = PICO_CE_FWD_UNROLL;   // pieces of the row requested together (bytes in flight per thread)
+  int v = threadIdx.x;
+  for (; v + (U - 1) * kThreads < nvec; v += U * kThreads) {
+    float e[U][V];
+#pragma unroll
+    for (int u = 0; u < U; ++u) load_as<T, PICO_NT_CE_FWD_LOADS != 0>(x + static_cast<int64_t>(v + u * kThreads) * V, e[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) absorb(e[u]);
+  }
+  for (; v < nvec; v += kThreads) {
+    float e[V];
+    load_as<T, PICO_NT_CE_FWD_LOADS != 0>(x + static_cast<int64_t>(v) * V, e);
+    absorb(e);
   }
   for (int j = nvec * V + threadIdx.x; j < vocab; j += kThreads) {  // tail when vocab is not a multiple of V
     const float e = static_cast<float>(x[j]) * kLog2e;
@@ -89,7 +107,27 @@ __global__ __launch_bounds__(kThreads) void ce_bwd_kernel(const T* __restrict__ 
   const float scale = (t != ignore_index && t >= 0 && t < vocab) ? *scale_ptr : 0.f;
   const float l2 = lse[row] * kLog2e;
   const int nvec = vocab / V;
-  for (int v = threadIdx.x; v < nvec; v += kThreads) {
+  // kCeUnroll pieces of the row per thread are requested before the first is used: one 16-byte load per thread at a
+  // time leaves too few bytes in flight to cover the memory latency
+  constexpr int U = PICO_CE_BWD_UNROLL;
+  int v = threadIdx.x;
+  for (; v + (U - 1) * kThreads < nvec; v += U * kThreads) {
+    float e[U][V];
+#pragma unroll
+    for (int u = 0; u < U; ++u) load_as<T, PICO_NT_CE_BWD_LOADS != 0>(x + static_cast<int64_t>(v + u * kThreads) * V, e[u]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      float o[V];
+      const int j0 = (v + u * kThreads) * V;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float p = fast_exp2(e[u][i] * kLog2e - l2);
+        o[i] = (p - ((j0 + i) == t ? 1.f : 0.f)) * scale;
+      }
+      store_as<T, PICO_NT_CE_BWD_STORES != 0>(d + static_cast<int64_t>(v + u * kThreads) * V, o);
+    }
+  }
+  for (; v < nvec; v += kThreads) {
     float e[V], o[V];
     load_as<T, PICO_NT_CE_BWD_LOADS != 0>(x + static_cast<int64_t>(v) * V, e);
     const int j0 = v * V;
