@@ -73,6 +73,18 @@ constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
 // -lse * log2e is what the S accumulator starts from, so the exponent comes out of the MFMA and the multiply-add in
 // front of every v_exp_f32 disappears (one of about seven vector instructions per score).  The scaled operand is
 // rounded to bf16 once more: an error of 2^-9 relative per element, i.e. of the size of the inputs' own rounding.
+#ifndef PICO_PAIR_KREGS
+#define PICO_PAIR_KREGS 4
+#endif
+#ifndef PICO_PAIR_STAGE_TOP
+#define PICO_PAIR_STAGE_TOP 1
+#endif
+#ifndef PICO_PAIR_AHEAD
+#define PICO_PAIR_AHEAD 1
+#endif
+#ifndef PICO_PAIR_AHEAD_T
+#define PICO_PAIR_AHEAD_T 2
+#endif
 #ifndef PICO_PRESCALE
 #define PICO_PRESCALE 1
 #endif
@@ -86,11 +98,16 @@ __device__ __forceinline__ void scale_fragments(bf16x8 (&f)[N], float c) {
     for (int e = 0; e < 8; ++e) f[s][e] = static_cast<__bf16>(static_cast<float>(f[s][e]) * c);
 }
 
-template <int D>
+// PAIR: eight waves instead of four; waves w and w + 4 (they share a SIMD) own the same 32 keys and split every
+// 64-query tile between them, one 32-query sub-block each, with accumulators of their own that are added through LDS
+// at the end of the key tile.  A wave then holds one sub-block's S / dP tiles instead of two, which is what lets the
+// head_dim 128 kernel fit 256 registers, i.e. two waves per SIMD.
+template <int D, bool PAIR = false>
 struct KvCfg {
-  static constexpr int NW = 4;
+  static constexpr int NW = PAIR ? 8 : 4;
+  static constexpr int kKeyWaves = 4;          // waves that own different keys
   static constexpr int kThreads = 64 * NW;
-  static constexpr int BN = 32 * NW;  // keys per workgroup
+  static constexpr int BN = 32 * kKeyWaves;  // keys per workgroup
   static constexpr int BM = 64;       // queries per trip
   // Q and dO tiles: rows of D elements at a pitch of LDQ elements, plus kSkew elements after every 4 rows.  Every
   // tile is read both by rows (16 bytes per lane, 32 consecutive rows per instruction) and transposed (8 bytes per
@@ -107,14 +124,20 @@ struct KvCfg {
   static constexpr int kQLoads = BM * kVecPerRow / kThreads;
   static constexpr int kBufElems = 2 * kTileElems;                     // Q + dO tile of one stage (bf16)
   static constexpr size_t kBufBytes = kBufElems * sizeof(__bf16) + 2 * BM * sizeof(float);
-  static constexpr size_t kLdsBytes = 2 * kBufBytes;                   // double-buffered
-  static_assert(NW * kRowRegionBytes <= kLdsBytes, "the epilogue reuses the tile buffers");
-  static_assert(NW * WaveTile<D>::kRegionBytes <= kBufBytes, "the K / V fragments pass through the second tile buffer");
+  static constexpr size_t kTileBytes = 2 * kBufBytes;  // the two Q / dO tile buffers
+  // PAIR: the K and V fragments of the four key waves stay in LDS behind the tile buffers instead of in registers
+  static constexpr size_t kKvBytes = PAIR ? static_cast<size_t>(kKeyWaves) * 2 * WaveTile<D>::kRegionBytes : 0;
+  static constexpr size_t kLdsBytes = kTileBytes + kKvBytes;
+  static_assert(NW * kRowRegionBytes <= kTileBytes, "the epilogue reuses the tile buffers");
+  static_assert(PAIR || NW * WaveTile<D>::kRegionBytes <= kBufBytes, "the K / V fragments pass through the second tile buffer");
+  // PAIR: one accumulator set (D/32 x 16 registers x 64 lanes of fp32) per key wave passes through LDS at a time
+  static constexpr size_t kPairExchangeBytes = static_cast<size_t>(D / 32) * 16 * 64 * 4;
+  static_assert(!PAIR || kKeyWaves * kPairExchangeBytes <= kTileBytes, "the pair exchange reuses the tile buffers");
 };
 
-template <int D>
+template <int D, bool PAIR = false>
 __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int ktile) {
-  using C = KvCfg<D>;
+  using C = KvCfg<D, PAIR>;
   constexpr int BM = C::BM, BN = C::BN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   auto tile_row = [](int r) { return r * C::LDQ + C::kSkew * (r >> 2); };   // element offset of a tile row
@@ -123,7 +146,10 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   const int hkv = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
   const int group = a.Hq / a.Hkv;
   const int key0 = ktile * BN;
-  const int tid = threadIdx.x, wave = tid / 64, lane = tid % 64;
+  const int tid = threadIdx.x, wave_id = tid / 64, lane = tid % 64;
+  // wave: which 32 keys of the tile; pair_sb (PAIR only): which 32-query sub-block of every query tile
+  const int wave = PAIR ? __builtin_amdgcn_readfirstlane(wave_id % C::kKeyWaves) : wave_id;
+  const int pair_sb = PAIR ? __builtin_amdgcn_readfirstlane(wave_id / C::kKeyWaves) : 0;
   const int n = lane % 32, h = lane / 32;
   const float c = a.sm_scale * kLog2e;
 
@@ -134,17 +160,37 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   //      row-major and turned into fragments through the wave's piece of the SECOND tile buffer, which nothing
   //      else writes before the end of the first trip, a barrier later
   bf16x8 kf[D / 16], vf[D / 16];
-  {
+  constexpr int kFragPitch = (D + 8) * 2;   // WaveTile's row pitch in bytes
+  unsigned char* const pair_k = smem_raw + C::kTileBytes + wave * 2 * WaveTile<D>::kRegionBytes;   // (PAIR only)
+  unsigned char* const pair_v = pair_k + WaveTile<D>::kRegionBytes;
+  if (!PAIR || pair_sb == 0) {
     // (the wave index read as a scalar: the buffer windows below are then built in scalar registers; from the
     // per-lane value the compiler cannot tell that they are the same in all lanes and loops over the lanes' values)
     const int row0 = key0 + 32 * __builtin_amdgcn_readfirstlane(wave);
     WaveTile<D> kt, vt;
     kt.issue(make_buffer(kbase + static_cast<int64_t>(row0) * a.ks[2], span_bytes(a.Sk - row0, a.ks[2], D)), a.ks[2], lane);
     vt.issue(make_buffer(vbase + static_cast<int64_t>(row0) * a.vs[2], span_bytes(a.Sk - row0, a.vs[2], D)), a.vs[2], lane);
-    unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
-    kt.fragments(region, lane, kf);
-    vt.fragments(region, lane, vf);
-    if constexpr (kPrescale) scale_fragments(kf, c);   // kf feeds the S product only (dK comes from Q^T dS)
+    if constexpr (!PAIR) {
+      unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
+      kt.fragments(region, lane, kf);
+      vt.fragments(region, lane, vf);
+      if constexpr (kPrescale) scale_fragments(kf, c);   // kf feeds the S product only (dK comes from Q^T dS)
+    } else {
+      // the first wave of each pair leaves both tiles in the pair's piece of LDS, K with the scale folded in
+      kt.fragments(pair_k, lane, kf);
+      if constexpr (kPrescale) {
+        scale_fragments(kf, c);
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) *reinterpret_cast<bf16x8*>(pair_k + n * kFragPitch + (16 * s + 8 * h) * 2) = kf[s];
+      }
+      vt.fragments(pair_v, lane, vf);
+    }
+  }
+  if constexpr (PAIR) {
+    __syncthreads();
+    // the first few K fragments stay in registers (as many as fit beside the accumulators)
+#pragma unroll
+    for (int j = 0; j < PICO_PAIR_KREGS; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
   }
 
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
@@ -252,6 +298,14 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   // of the NEXT tile on every trip.
   __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
   __syncthreads();
+  // PAIR (PICO_PAIR_STAGE_TOP): the tile after the one being computed goes to LDS at the TOP of a trip, from loads that
+  // were issued at the top of the trip before; the registers are then reloaded with the tile after that.  The LDS
+  // writes are off the end of the trip (where every wave of the workgroup would wait for them in front of the barrier)
+  // and a load has a whole trip to arrive.
+  constexpr bool kStageTop = PAIR && PICO_PAIR_STAGE_TOP != 0;
+  if constexpr (kStageTop) {
+    if (n_iter > 1) { advance(); prefetch(); }
+  }
 
   const int kw0 = key0 + 32 * wave;
   int tile = qt_start;       // query tile (within its head) of the trip being computed
@@ -260,7 +314,14 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     // tile it+1 travels global -> registers while this trip computes; it goes to the other LDS buffer at
     // the end of the trip (that buffer's readers finished before the barrier that ended trip it-1)
     const bool has_next = it + 1 < n_iter;
-    if (has_next) advance();
+    if constexpr (kStageTop) {
+      if (has_next) {
+        stage(buf_off == 0);   // tile it+1 (the cursor is on it)
+        if (it + 2 < n_iter) { advance(); prefetch(); }
+      }
+    } else {
+      if (has_next) advance();
+    }
     const int q0 = tile * BM;
     const __bf16* sQ = reinterpret_cast<const __bf16*>(smem_raw + buf_off);
     const __bf16* sdO = sQ + C::kTileElems;
@@ -279,12 +340,36 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 #pragma unroll
         for (int t = 0; t < 4; ++t) { s_acc[4 * j + t] = s4[t]; dp_acc[4 * j + t] = d4[t]; }
       }
+      if constexpr (PAIR) {
+        // both operands of every MFMA come from LDS: they are requested kAhead steps before the MFMAs that use them, and
+        // the scheduling barriers keep that order (left alone, the compiler reuses one set of registers and every MFMA
+        // waits for an LDS round trip)
+        constexpr int kSteps = D / 16, kAhead = PICO_PAIR_AHEAD;
+        bf16x8 qa[kSteps], da[kSteps], kb[kSteps], vb[kSteps];
+        auto fetch = [&](int j) {
+          qa[j] = *reinterpret_cast<const bf16x8*>(&sQ[tile_row(32 * sb + n) + 16 * j + 8 * h]);
+          if (j >= PICO_PAIR_KREGS) kb[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
+          da[j] = *reinterpret_cast<const bf16x8*>(&sdO[tile_row(32 * sb + n) + 16 * j + 8 * h]);
+          vb[j] = *reinterpret_cast<const bf16x8*>(pair_v + n * kFragPitch + (16 * j + 8 * h) * 2);
+        };
 #pragma unroll
-      for (int s = 0; s < D / 16; ++s) {
-        const bf16x8 qa = *reinterpret_cast<const bf16x8*>(&sQ[tile_row(32 * sb + n) + 16 * s + 8 * h]);
-        const bf16x8 da = *reinterpret_cast<const bf16x8*>(&sdO[tile_row(32 * sb + n) + 16 * s + 8 * h]);
-        s_acc = mfma32(qa, kf[s], s_acc);
-        dp_acc = mfma32(da, vf[s], dp_acc);
+        for (int j = 0; j < kAhead; ++j) fetch(j);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int j = 0; j < kSteps; ++j) {
+          if (j + kAhead < kSteps) fetch(j + kAhead);
+          s_acc = mfma32(qa[j], j < PICO_PAIR_KREGS ? kf[j] : kb[j], s_acc);
+          dp_acc = mfma32(da[j], vb[j], dp_acc);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      } else {
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) {
+          const bf16x8 qa = *reinterpret_cast<const bf16x8*>(&sQ[tile_row(32 * sb + n) + 16 * s + 8 * h]);
+          const bf16x8 da = *reinterpret_cast<const bf16x8*>(&sdO[tile_row(32 * sb + n) + 16 * s + 8 * h]);
+          s_acc = mfma32(qa, kf[s], s_acc);
+          dp_acc = mfma32(da, vf[s], dp_acc);
+        }
       }
     };
     // softmax_grad(): P = exp2(S*c - lse*log2e), dS = P * (dP - delta) [already in the accumulator]; the mask test
@@ -313,6 +398,31 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     // d, which is what lets the epilogue write whole 16-byte pieces of a row); P / dS come from the registers,
     // dO^T / Q^T from the row-major LDS tiles through transposing reads.
     auto accumulate = [&](int sb, const f32x16& s_acc, const f32x16& dp_acc) {
+      if constexpr (PAIR) {
+        constexpr int kSlots = 2 * (D / 32), kAhead = PICO_PAIR_AHEAD_T;
+        bf16x8 dof[kSlots], qf[kSlots];
+        auto fetch = [&](int idx) {
+          const int cc = idx / (D / 32), db = idx % (D / 32);
+          const int qr = 32 * sb + 16 * cc + 4 * h + (lane % 16) / 4;
+          const int col = 32 * db + 16 * ((lane / 16) % 2) + 4 * (lane % 4);
+          dof[idx] = lds_read_tr_pair_step(&sdO[tile_row(qr) + col], C::kTrStep);
+          qf[idx] = lds_read_tr_pair_step(&sQ[tile_row(qr) + col], C::kTrStep);
+        };
+#pragma unroll
+        for (int j = 0; j < kAhead; ++j) fetch(j);
+        bf16x8 pf = pack8(s_acc, 0), dsf = pack8(dp_acc, 0);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int idx = 0; idx < kSlots; ++idx) {
+          const int db = idx % (D / 32);
+          if (idx + kAhead < kSlots) fetch(idx + kAhead);
+          dv_acc[db] = mfma32(dof[idx], pf, dv_acc[db]);
+          dk_acc[db] = mfma32(qf[idx], dsf, dk_acc[db]);
+          if (idx + 1 == D / 32) { pf = pack8(s_acc, 8); dsf = pack8(dp_acc, 8); }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        return;
+      }
 #pragma unroll
       for (int cc = 0; cc < 2; ++cc) {
         // registers 8cc+4jj+t hold queries 32sb + 16cc + 8jj + 4h + t: fetch dO / Q rows in that order
@@ -330,8 +440,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
     };
 
-    const bool off_diagonal = kPipelineTrip && BM == 64 && (!a.causal || kw0 + 31 <= a.q_offset + q0);
-    if (has_next && !off_diagonal) prefetch();
+    const bool off_diagonal = !PAIR && kPipelineTrip && BM == 64 && (!a.causal || kw0 + 31 <= a.q_offset + q0);
+    if (!kStageTop && has_next && !off_diagonal) prefetch();
     if (off_diagonal) {
       // Every pair of this trip is visible to this wave (all trips off the diagonal): straight-line code in an order
       // that lets the wave's own phases overlap -- the matrix pipe works on the second sub-block's S / dP while the
@@ -446,7 +556,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
     } else {
 #pragma unroll
-      for (int sb = 0; sb < BM / 32; ++sb) {
+      for (int sbi = 0; sbi < (PAIR ? 1 : BM / 32); ++sbi) {
+        const int sb = PAIR ? pair_sb : sbi;
         const int qs_pos = a.q_offset + q0 + 32 * sb;       // position of the sub-block's first query
         if (a.causal && kw0 > qs_pos + 31) continue;        // every (query, key) pair of this block is masked
         f32x16 s_acc, dp_acc;
@@ -457,7 +568,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
     }
     buf_off ^= static_cast<uint32_t>(C::kBufBytes);
-    if (has_next) stage(buf_off != 0);
+    if (!kStageTop && has_next) stage(buf_off != 0);
     tile = tile + 1 == n_qtiles ? qt_start : tile + 1;
     __syncthreads();  // all waves are done with the buffer just read (refilled in the next trip) and the next tile is visible
   }
@@ -465,7 +576,34 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   // ---- epilogue: dK (scaled) and dV rows of this wave's 32 keys, through the wave's piece of LDS (free now:
   //      the loop ended on a barrier).  bf16 gradients are written with streaming stores: nothing on this
   //      GPU reads them back soon, and lines left dirty in L2 are only written back when the kernel ends.
-  {
+  if constexpr (PAIR) {
+    // the second wave of each pair hands its sums over, dK then dV (the loop ended on a barrier, or never ran)
+    float* xch = reinterpret_cast<float*>(smem_raw + wave * C::kPairExchangeBytes);
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+      f32x16 (&acc)[D / 32] = which == 0 ? dk_acc : dv_acc;
+      if (pair_sb == 1) {
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; i += 4)
+            *reinterpret_cast<f32x4*>(&xch[((db * 4 + i / 4) * 64 + lane) * 4]) = f32x4{acc[db][i], acc[db][i + 1], acc[db][i + 2], acc[db][i + 3]};
+      }
+      __syncthreads();
+      if (pair_sb == 0) {
+#pragma unroll
+        for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+          for (int i = 0; i < 16; i += 4) {
+            const f32x4 o = *reinterpret_cast<const f32x4*>(&xch[((db * 4 + i / 4) * 64 + lane) * 4]);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc[db][i + t] += o[t];
+          }
+      }
+      __syncthreads();
+    }
+  }
+  if (!PAIR || pair_sb == 0) {
     unsigned char* region = smem_raw + wave * kRowRegionBytes;
     const int row0 = key0 + 32 * wave;
     const int rows_live = a.Sk - row0;
@@ -488,15 +626,15 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 // workgroup takes tile t and then tile n-1-t: under a causal mask every pair is the same amount of work, so a
 // launch whose pairs fill the GPU once ends without a tail of short workgroups and pays the start-up of a
 // workgroup (kernel arguments, first loads) half as often.
-template <int D>
+template <int D, bool PAIR = false>
 __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
-  const int n_ktiles = (p.a.Sk + KvCfg<D>::BN - 1) / KvCfg<D>::BN;
+  const int n_ktiles = (p.a.Sk + KvCfg<D, PAIR>::BN - 1) / KvCfg<D, PAIR>::BN;
   const int first = blockIdx.y;
-  attn_bwd_dkdv_tile<D>(p, first);
+  attn_bwd_dkdv_tile<D, PAIR>(p, first);
   const int second = n_ktiles - 1 - first;
   if (p.pair_ktiles && second != first) {
     __syncthreads();  // the epilogue's pieces of LDS are the next tile's buffers
-    attn_bwd_dkdv_tile<D>(p, second);
+    attn_bwd_dkdv_tile<D, PAIR>(p, second);
   }
 }
 
@@ -505,7 +643,12 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_dkdv_kernel_d64(const BwdParams p) {
   attn_bwd_dkdv_body<64>(p);
 }
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel_d128(const BwdParams p) { attn_bwd_dkdv_body<128>(p); }
+#ifndef PICO_DKDV_PAIR128
+#define PICO_DKDV_PAIR128 1
+#endif
+__global__ __launch_bounds__(PICO_DKDV_PAIR128 ? 512 : 256) void attn_bwd_dkdv_kernel_d128(const BwdParams p) {
+  attn_bwd_dkdv_body<128, PICO_DKDV_PAIR128 != 0>(p);
+}
 
 template <int D> struct KvKernel;
 template <> struct KvKernel<64> { static constexpr auto fn = &attn_bwd_dkdv_kernel_d64; };
@@ -822,7 +965,7 @@ __global__ __launch_bounds__(256) void attn_bwd_preprocess_kernel(const __bf16* 
 
 template <int D>
 int launch_dkdv(const BwdParams& p, hipStream_t s) {
-  using C = KvCfg<D>;
+  using C = KvCfg<D, D == 128 && PICO_DKDV_PAIR128 != 0>;
   static std::atomic<bool> lds_reserved{false};
   if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(KvKernel<D>::fn), C::kLdsBytes))
     return fail(PICO_ERR_LAUNCH, "pico_attn_bwd(dk/dv): cannot reserve %zu bytes of LDS", C::kLdsBytes);
