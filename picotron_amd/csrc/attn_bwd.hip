@@ -158,39 +158,20 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 
   // ---- K, V fragments of this wave's 32 keys (B operand: lane = key, 8 consecutive d per k step), fetched
   //      row-major and turned into fragments through the wave's piece of the SECOND tile buffer, which nothing
-  //      else writes before the end of the first trip, a barrier later
+  //      else writes before the end of the first trip, a barrier later.  The loads are issued here; the first
+  //      Q / dO tile's loads follow them further down before anything waits, so that the two latencies overlap.
   bf16x8 kf[D / 16], vf[D / 16];
   constexpr int kFragPitch = (D + 8) * 2;   // WaveTile's row pitch in bytes
   unsigned char* const pair_k = smem_raw + C::kTileBytes + wave * 2 * WaveTile<D>::kRegionBytes;   // (PAIR only)
   unsigned char* const pair_v = pair_k + WaveTile<D>::kRegionBytes;
-  if (!PAIR || pair_sb == 0) {
+  const bool loads_kv = !PAIR || pair_sb == 0;
+  WaveTile<D> kt, vt;
+  if (loads_kv) {
     // (the wave index read as a scalar: the buffer windows below are then built in scalar registers; from the
     // per-lane value the compiler cannot tell that they are the same in all lanes and loops over the lanes' values)
     const int row0 = key0 + 32 * __builtin_amdgcn_readfirstlane(wave);
-    WaveTile<D> kt, vt;
     kt.issue(make_buffer(kbase + static_cast<int64_t>(row0) * a.ks[2], span_bytes(a.Sk - row0, a.ks[2], D)), a.ks[2], lane);
     vt.issue(make_buffer(vbase + static_cast<int64_t>(row0) * a.vs[2], span_bytes(a.Sk - row0, a.vs[2], D)), a.vs[2], lane);
-    if constexpr (!PAIR) {
-      unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
-      kt.fragments(region, lane, kf);
-      vt.fragments(region, lane, vf);
-      if constexpr (kPrescale) scale_fragments(kf, c);   // kf feeds the S product only (dK comes from Q^T dS)
-    } else {
-      // the first wave of each pair leaves both tiles in the pair's piece of LDS, K with the scale folded in
-      kt.fragments(pair_k, lane, kf);
-      if constexpr (kPrescale) {
-        scale_fragments(kf, c);
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) *reinterpret_cast<bf16x8*>(pair_k + n * kFragPitch + (16 * s + 8 * h) * 2) = kf[s];
-      }
-      vt.fragments(pair_v, lane, vf);
-    }
-  }
-  if constexpr (PAIR) {
-    __syncthreads();
-    // the first few K fragments stay in registers (as many as fit beside the accumulators)
-#pragma unroll
-    for (int j = 0; j < PICO_PAIR_KREGS; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
   }
 
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
@@ -290,8 +271,31 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   if (n_iter > 0) {
     seek(hkv * group, qt_start);
     prefetch();
-    stage(0);
   }
+  if (loads_kv) {
+    if constexpr (!PAIR) {
+      unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
+      kt.fragments(region, lane, kf);
+      vt.fragments(region, lane, vf);
+      if constexpr (kPrescale) scale_fragments(kf, c);   // kf feeds the S product only (dK comes from Q^T dS)
+    } else {
+      // the first wave of each pair leaves both tiles in the pair's piece of LDS, K with the scale folded in
+      kt.fragments(pair_k, lane, kf);
+      if constexpr (kPrescale) {
+        scale_fragments(kf, c);
+#pragma unroll
+        for (int s = 0; s < D / 16; ++s) *reinterpret_cast<bf16x8*>(pair_k + n * kFragPitch + (16 * s + 8 * h) * 2) = kf[s];
+      }
+      vt.fragments(pair_v, lane, vf);
+    }
+  }
+  if constexpr (PAIR) {
+    __syncthreads();
+    // the first few K fragments stay in registers (as many as fit beside the accumulators)
+#pragma unroll
+    for (int j = 0; j < PICO_PAIR_KREGS; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
+  }
+  if (n_iter > 0) stage(0);
   // The K / V fragment loads above are complete by now on every path that enters the loop (the LDS fill
   // waited for all loads), but not on the static path that skips the fill; saying so here keeps the compiler
   // from putting a vmcnt(0) wait in front of the loop's first MFMAs, where it would wait for the prefetch
