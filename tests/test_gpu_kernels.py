@@ -385,6 +385,39 @@ def test_attn_bwd_paired_key_tiles_match_unpaired(ops, device):
     assert rel_l2(whole[1][:1, :1], gk) <= 1e-2 and rel_l2(whole[2][:1, :1], gv) <= 1e-2 and rel_l2(whole[0][:1, :1], gq) <= 1e-2
 
 
+def test_attn_bwd_head_dim_128_wave_pairs(ops, device):
+    """head_dim 128: two waves share a 32-key block of the dK/dV kernel, take one 32-query sub-block each and add their
+    partial dK / dV through LDS at the end of a key tile.  Two runs are bit-identical; a launch big enough for paired key
+    tiles (t and n-1-t in one workgroup; odd tile count, ragged last tile) equals the launches of half the batch, which
+    take one tile per workgroup; fp32 outputs with accumulate add to what is there; one head against the oracle."""
+    B, H, S, D = 4, 16, 1100, 128
+    scale = 1 / math.sqrt(D)
+    q, k, v = (t.to(device) for t in attn_inputs(B, H, H, S, S, D, seed=95))
+    do = rnd(B, H, S, D, seed=96).to(torch.bfloat16).to(device)
+    out, lse = ops.attn_fwd(q, k, v, scale, True)
+    delta = ops.attn_bwd_preprocess(do, out)
+    whole = ops.attn_bwd(do, q, k, v, lse, delta, scale, True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16)
+    again = ops.attn_bwd(do, q, k, v, lse, delta, scale, True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16)
+    for x, y in zip(whole, again):
+        assert torch.equal(x, y)
+    for half in (slice(0, 2), slice(2, 4)):
+        part = ops.attn_bwd(do[half], q[half], k[half], v[half], lse[half].contiguous(), delta[half].contiguous(), scale,
+                            True, 0, dq_dtype=torch.bfloat16, dkv_dtype=torch.bfloat16)
+        for x, y in zip(whole, part):
+            assert torch.equal(x[half], y)
+    # fp32 dk / dv added to what the buffers hold
+    dk = torch.full((B, H, S, D), 2.0, dtype=torch.float32, device=device)
+    dv = torch.full((B, H, S, D), -1.0, dtype=torch.float32, device=device)
+    ops.attn_bwd(do, q, k, v, lse, delta, scale, True, 0, None, dk, dv, want_dq=False, dkv_accumulate=True)
+    plain = ops.attn_bwd(do, q, k, v, lse, delta, scale, True, 0, want_dq=False)
+    assert (dk - 2.0 - plain[1]).abs().max().item() <= 1e-5 * plain[1].abs().max().item() + 1e-6
+    assert (dv + 1.0 - plain[2]).abs().max().item() <= 1e-5 * plain[2].abs().max().item() + 1e-6
+    qf, kf, vf = (t[:1, :1].float().cpu().requires_grad_() for t in (q, k, v))
+    w_o, _ = OR.full_attention_closed_form(qf, kf, vf, scale, True, 0)
+    gq, gk, gv = torch.autograd.grad(w_o, (qf, kf, vf), do[:1, :1].float().cpu())
+    assert rel_l2(whole[1][:1, :1], gk) <= 1e-2 and rel_l2(whole[2][:1, :1], gv) <= 1e-2 and rel_l2(whole[0][:1, :1], gq) <= 1e-2
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Sk,D,causal,q_offset", [
     (2, 4, 4, 300, 300, 64, True, 0), (1, 4, 2, 128, 384, 128, True, 256), (1, 2, 1, 77, 203, 64, False, 0)])
 def test_attn_bwd_with_delta_computed_inside(ops, device, B, Hq, Hkv, Sq, Sk, D, causal, q_offset):
