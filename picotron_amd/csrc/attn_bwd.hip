@@ -970,7 +970,7 @@ __global__ __launch_bounds__(256) void attn_bwd_preprocess_kernel(const __bf16* 
 template <int D>
 int launch_dkdv(const BwdParams& p, hipStream_t s) {
   using C = KvCfg<D, D == 128 && PICO_DKDV_PAIR128 != 0>;
-  static std::atomic<bool> lds_reserved{false};
+  static LdsOnce lds_reserved;
   if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(KvKernel<D>::fn), C::kLdsBytes))
     return fail(PICO_ERR_LAUNCH, "pico_attn_bwd(dk/dv): cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_ktiles = (p.a.Sk + C::BN - 1) / C::BN;
@@ -986,7 +986,7 @@ int launch_dkdv(const BwdParams& p, hipStream_t s) {
 template <int D, int NW, int KT, bool kDelta, int KS>
 int launch_dq_impl(const BwdParams& p, hipStream_t s) {
   using C = DqCfg<D, NW, KT, KS>;
-  static std::atomic<bool> lds_reserved{false};
+  static LdsOnce lds_reserved;
   if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(&attn_bwd_dq_kernel<D, NW, KT, kDelta, KS>), C::kLdsBytes))
     return fail(PICO_ERR_LAUNCH, "pico_attn_bwd(dq): cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;

@@ -425,7 +425,7 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
 template <int D, int QB, int NW, int KT, int KS = 1>
 int launch(const FwdParams& p, hipStream_t s) {
   using C = FwdCfg<D, QB, NW, KT, KS>;
-  static std::atomic<bool> lds_reserved{false};
+  static LdsOnce lds_reserved;
   if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(&attn_fwd_kernel<D, QB, NW, KT, KS>), C::kLdsBytes))
     return fail(PICO_ERR_LAUNCH, "pico_attn_fwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;

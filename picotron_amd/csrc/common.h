@@ -128,14 +128,22 @@ __device__ __forceinline__ void store_as(void* p, const float (&in)[N]) {
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Raises a kernel's dynamic-LDS limit the first time the kernel is launched.  Host threads may race here (autograd
-// runs backward on a thread of its own): the flag is atomic and the HIP call is idempotent, so two first callers
-// both make it and both proceed only after it has succeeded.
-inline bool reserve_lds_once(std::atomic<bool>& done, const void* kernel, size_t bytes) {
-  if (done.load(std::memory_order_acquire)) return true;
+// Raises a kernel's dynamic-LDS limit the first time the kernel is launched on a device (the attribute belongs to the
+// kernel's code object on that device, so a process that drives several GPUs sets it once on each).  Host threads may
+// race here (autograd runs backward on a thread of its own): the per-device bits are atomic and the HIP call is
+// idempotent, so two first callers both make it and both proceed only after it has succeeded.
+struct LdsOnce {
+  std::atomic<uint64_t> devices{0};   // bit d: done on device d (devices 64 and up set the attribute on every launch)
+};
+inline bool reserve_lds_once(LdsOnce& once, const void* kernel, size_t bytes) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const bool tracked = dev >= 0 && dev < 64;
+  const uint64_t bit = tracked ? (uint64_t{1} << dev) : 0;
+  if (tracked && (once.devices.load(std::memory_order_acquire) & bit)) return true;
   if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(bytes)) != hipSuccess)
     return false;
-  done.store(true, std::memory_order_release);
+  if (tracked) once.devices.fetch_or(bit, std::memory_order_release);
   return true;
 }
 

@@ -418,7 +418,7 @@ int launch_bwd(const void* dy, const void* x, const void* w, const float* rstd, 
                float* partial, int blocks, int64_t rows, int hidden, hipStream_t s) {
   const size_t lds = (kBwdThreads / G > 1) ? static_cast<size_t>(hidden) * sizeof(float) : 0;
   // the longest rows need the whole default LDS allowance for the dweight row plus the kernel's static 32 bytes
-  static std::atomic<bool> lds_reserved{false};
+  static LdsOnce lds_reserved;
   constexpr size_t kLdsMax = static_cast<size_t>(G) * NV * io<T>::kVec * sizeof(float) + 64;
   if (kLdsMax > 48 * 1024 &&
       !reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(&rmsnorm_bwd_kernel<T, G, NV>), kLdsMax))
@@ -469,7 +469,7 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
     const int blocks = bwd_blocks(rows, kBwdWaves, hidden);                                            \
     *blocks_out = blocks;                                                                              \
     const size_t lds = static_cast<size_t>(kBwdWaves) * hidden * sizeof(float);                        \
-    auto go = [&](auto kern, std::atomic<bool>& reserved) -> int {                                     \
+    auto go = [&](auto kern, LdsOnce& reserved) -> int {                                               \
       if (lds > 48 * 1024 && !reserve_lds_once(reserved, reinterpret_cast<const void*>(kern),          \
                                                kBwdWaves * 64 * NV * io<T>::kVec * sizeof(float)))     \
         return fail(PICO_ERR_LAUNCH, "pico_rmsnorm_bwd: cannot reserve %zu bytes of LDS", lds);        \
@@ -478,7 +478,7 @@ int dispatch_bwd(const void* dy, const void* x, const void* w, const float* rstd
                          rstd, static_cast<const T*>(dres), static_cast<T*>(dx), partial, rows, hidden); \
       return PICO_OK;                                                                                  \
     };                                                                                                 \
-    static std::atomic<bool> reserved_res{false}, reserved_res2{false}, reserved_plain{false};                               \
+    static LdsOnce reserved_res, reserved_res2, reserved_plain;                               \
     /* with dresidual and short rows a wave that owns several rows keeps two in flight (measured at 4096 x 2048: \
        20.2 -> 18.8 us; without dresidual the same costs 0.9 us, with longer rows the registers do not allow it) */ \
     constexpr int kR = NV * io<T>::kVec <= 32 ? 2 : 1;                                                 \
