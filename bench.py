@@ -214,6 +214,21 @@ class RingBench:
         self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
 
 
+def seq_len_extra(torch, ops, iters=10):
+    """The headline step (one causal forward + backward launch set over whole sequences, head_dim 64, 32 heads) at the
+    same 4096 tokens but longer sequences: configs[1]'s launches are one generation of workgroups whose loads and stores
+    are not hidden behind anyone's matrix work; with more trips per workgroup that share shrinks."""
+    out = {}
+    for B, S in ((4, 1024), (2, 2048), (1, 4096), (1, 8192)):
+        rb = RingBench(torch, ops, B=B, S=S, W=1)
+        fwd_flops, bwd_flops = rb.flops()
+        ms, _ = graph_time(torch, rb.step_batched, iters, per_graph=5)
+        out[f"B{B}_S{S}"] = {"ms_per_step": round(ms, 4), "TFLOP/s": round((fwd_flops + bwd_flops) / (ms * 1e-3) / 1e12, 1),
+                            "frac_of_mfma_peak": round((fwd_flops + bwd_flops) / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del rb
+    return out
+
+
 def preheat(torch, launch, seconds=0.1, batch=10):
     """Untimed launches for `seconds` of wall-clock, ending on a synchronize.  The GPU's clocks follow its load with a
     delay: after an idle stretch (a graph capture, host-side set-up) the first tens of milliseconds of work run about
@@ -648,6 +663,7 @@ def main():
         extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4),
                                               "frac_of_mfma_peak": round(total_flops / (ms_ring * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                               "schedule": "the reference's shape: block + fused merge per ring step, ranks and steps in sequence"}
+        extras["same_step_at_longer_sequences"] = seq_len_extra(torch, ops)
         extras["bandwidth_kernels"] = bandwidth_extras(torch, ops)
         extras["configs4_long_context_rank7_of_8"] = long_context_extra(torch, ops)
         if not args.no_train:
