@@ -93,3 +93,44 @@ def test_layer_sized_call_sequence_replays_like_eager_launches(device, D, Hq, Hk
         torch.cuda.synchronize()
         for name, t in recorded.items():
             assert torch.equal(t, eager[name]), f"replay {replay}: {name} differs from the eager result"
+
+
+def test_calls_from_several_host_threads_on_their_own_streams(device):
+    """The library keeps no mutable state between calls (its last-error text is per thread, its once-only set-up
+    is atomic): four host threads, each with a stream of its own, run the forward and backward repeatedly and get the
+    results of a single-threaded run bit for bit (autograd calls backward from a thread of its own)."""
+    import threading
+    from picotron_amd import ops
+    B, H, S, D = 2, 8, 384, 64
+    scale = 1 / math.sqrt(D)
+    bf = torch.bfloat16
+    cases = []
+    for t in range(4):
+        q, k, v, do = (rnd(B, H, S, D, seed=20 + 4 * t + i).to(bf).to(device) for i in range(4))
+        out, lse = ops.attn_fwd(q, k, v, scale, True)
+        grads = ops.attn_bwd(do, q, k, v, lse, None, scale, True, 0, dq_dtype=bf, dkv_dtype=bf, out=out)
+        cases.append((q, k, v, do, out, lse, grads))
+    torch.cuda.synchronize()
+    errors = []
+
+    def worker(t):
+        try:
+            q, k, v, do, out0, lse0, grads0 = cases[t]
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(20):
+                    out, lse = ops.attn_fwd(q, k, v, scale, True)
+                    grads = ops.attn_bwd(do, q, k, v, lse, None, scale, True, 0, dq_dtype=bf, dkv_dtype=bf, out=out)
+                stream.synchronize()
+            ok = torch.equal(out, out0) and torch.equal(lse, lse0) and all(torch.equal(a, b) for a, b in zip(grads, grads0))
+            if not ok:
+                errors.append(f"thread {t}: results differ from the single-threaded run")
+        except Exception as e:  # noqa: BLE001 -- reported by the main thread
+            errors.append(f"thread {t}: {e!r}")
+
+    threads = [threading.Thread(target=worker, args=(t,)) for t in range(4)]
+    for th in threads:
+        th.start()
+    for th in threads:
+        th.join()
+    assert not errors, errors
