@@ -70,8 +70,9 @@ int64_t pico_rmsnorm_bwd_workspace_bytes(int64_t rows, int64_t hidden);
  * dresidual: optional [rows, hidden] `dtype`, added to dx -- the gradient that reached the residual stream directly
  *   when the forward fused the residual add (the dresidual input of layer_norm_fn's backward); dx may alias it.
  * dx: [rows, hidden] `dtype` (may alias dy); dweight: [hidden] of dweight_dtype (PICO_F32 or PICO_BF16; summed in fp32
- *   and rounded once); workspace: device scratch of at least pico_rmsnorm_bwd_workspace_bytes() bytes (contents
- *   undefined on entry and exit).
+ *   and rounded once, the rows' contributions always in the same order: no atomics, equal inputs give equal bits);
+ *   workspace: device scratch of at least pico_rmsnorm_bwd_workspace_bytes() bytes (contents undefined on entry and
+ *   exit).
  */
 int pico_rmsnorm_bwd(const void* dy, const void* x, const void* weight, const float* rstd, const void* dresidual,
                      void* dx, void* dweight, int dweight_dtype, void* workspace, int64_t workspace_bytes,

@@ -179,13 +179,19 @@ __global__ __launch_bounds__(kBwdThreads) void rmsnorm_bwd_kernel(
   }
   float* out = partial + static_cast<int64_t>(blockIdx.x) * hidden;
   if constexpr (GPB > 1) {
-    __syncthreads();
+    // the groups of the block add their shares one after the other, in group order: the same sum on every run
+    // (an atomic add per element would take them in arrival order)
+    for (int turn = 0; turn < GPB; ++turn) {
+      __syncthreads();
+      if (gid == turn) {
 #pragma unroll
-    for (int j = 0; j < NV; ++j) {
-      const int v = t + j * G;
-      if (v < nvec) {
+        for (int j = 0; j < NV; ++j) {
+          const int v = t + j * G;
+          if (v < nvec) {
 #pragma unroll
-        for (int e = 0; e < V; ++e) atomicAdd(&dw_lds[v * V + e], dw[j][e]);
+            for (int e = 0; e < V; ++e) dw_lds[v * V + e] += dw[j][e];
+          }
+        }
       }
     }
     __syncthreads();

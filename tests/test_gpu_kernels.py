@@ -102,6 +102,21 @@ def test_rmsnorm_bwd_adds_residual_gradient_and_rounds_dweight(ops, device, rows
         assert ((dx.double().cpu() - exact).abs() <= exact.abs() * 2.0 ** -8 + want_dx.double().abs() * 2.0 ** -7 + 1e-6).all()
 
 
+def test_rmsnorm_bwd_is_bit_reproducible_at_every_row_length_class(ops, device):
+    """dweight is summed without atomics: two runs give the same bits, for the row-per-wave kernels, for the rows a
+    256-thread group owns (two groups per block meet in LDS, in group order) and for the longest rows."""
+    for rows, hidden, dtype in ((1000, 2048, torch.bfloat16), (1000, 4096, torch.bfloat16), (700, 8192, torch.bfloat16),
+                                (300, 16384, torch.bfloat16), (500, 8192, torch.float32), (900, 1000, torch.float32)):
+        x = rnd(rows, hidden, seed=70, dtype=dtype).to(device)
+        dy = rnd(rows, hidden, seed=71, dtype=dtype).to(device)
+        w = (1 + 0.1 * rnd(hidden, seed=72)).to(dtype).to(device)
+        _, rstd, _ = ops.rmsnorm_fwd(x, w, 1e-5, False)
+        a = ops.rmsnorm_bwd(dy, x, w, rstd)
+        for _ in range(3):
+            b = ops.rmsnorm_bwd(dy, x, w, rstd)
+            assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1]), (rows, hidden, dtype)
+
+
 # ------------------------------------------------------------------------------------ RoPE
 @pytest.mark.parametrize("B,H,S,D", [(2, 3, 17, 64), (1, 4, 33, 128), (1, 2, 5, 16)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
