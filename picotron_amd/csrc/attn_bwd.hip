@@ -1092,9 +1092,13 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     if (desc->D == 64) {
       auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
+      const int64_t visible_keys = desc->causal ? std::min<int64_t>(desc->Sk, static_cast<int64_t>(desc->q_offset) + desc->Sq) : desc->Sk;
       if (groups(256) >= PICO_DQ_NW8_MIN) rc = launch_dq<64, 8, 64>(p, s);
       else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
-      else rc = launch_dq<64, 4, 128, 2>(p, s);   // few waves in all: two waves per 32 queries, 64 keys of every 128 each
+      // few waves in all: two waves per 32 queries, 64 keys of every 128 each -- eight waves per workgroup under the
+      // forward's conditions (rank 3 of 4 at configs[1]: 18.8 -> 17.9 us)
+      else if (groups(128) >= 256 && visible_keys >= 512) rc = launch_dq<64, 8, 128, 2>(p, s);
+      else rc = launch_dq<64, 4, 128, 2>(p, s);
     } else {
       if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch_dq<128, 8, 64>(p, s);
       else rc = launch_dq<128, 4, 64>(p, s);
