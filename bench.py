@@ -129,9 +129,9 @@ class RingBench:
         ops = self.ops
         q, k, v, do, out, dk, dv = self._views(r)
         ops.attn_fwd(q, k, v, self.scale, True, r * self.Sc, out=out, lse=self.lse[r])
-        delta = ops.attn_bwd_preprocess(do, out, delta=self.delta[r])
-        ops.attn_bwd(do, q, k, v, self.lse[r], delta, self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
-                     dkv_accumulate=True)
+        # (one block per rank in this schedule, so delta = sum_d dO * O is computed in the dQ kernel's prologue)
+        ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
+                     dkv_accumulate=True, out=out)
 
     def step_ranks_parallel(self):
         """One launch per rank and direction, like step(), but the ranks' launches are independent branches: rank r's
