@@ -1093,11 +1093,17 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
     if (desc->D == 64) {
       auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
       const int64_t visible_keys = desc->causal ? std::min<int64_t>(desc->Sk, static_cast<int64_t>(desc->q_offset) + desc->Sq) : desc->Sk;
+      // the forward's rules: eight waves per workgroup also for rectangular launches (every query sees at least as many
+      // keys as there are queries) with fewer workgroups than the square ones need
+      const bool rectangular = !desc->causal || desc->q_offset >= desc->Sq;
       if (groups(256) >= PICO_DQ_NW8_MIN) rc = launch_dq<64, 8, 64>(p, s);
-      else if (groups(128) >= 512) rc = launch_dq<64, 4, 64>(p, s);
-      // few waves in all: two waves per 32 queries, 64 keys of every 128 each -- eight waves per workgroup under the
-      // forward's conditions (rank 3 of 4 at configs[1]: 18.8 -> 17.9 us)
-      else if (groups(128) >= 256 && visible_keys >= 512) rc = launch_dq<64, 8, 128, 2>(p, s);
+      else if (groups(128) >= 512) {
+        if (rectangular && groups(256) >= 256) rc = launch_dq<64, 8, 64>(p, s);
+        else rc = launch_dq<64, 4, 64>(p, s);
+      }
+      // few waves in all: two waves per 32 queries, 64 keys of every 128 each (rank 3 of 4 at configs[1] with eight waves
+      // per workgroup: 18.8 -> 17.9 us)
+      else if (groups(128) >= 256 && rectangular && visible_keys >= 512) rc = launch_dq<64, 8, 128, 2>(p, s);
       else rc = launch_dq<64, 4, 128, 2>(p, s);
     } else {
       if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch_dq<128, 8, 64>(p, s);

@@ -535,12 +535,20 @@ int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
     auto groups = [&](int bm) { return heads * ((desc->Sq + bm - 1) / bm); };
     const int64_t visible_keys = desc->causal ? std::min<int64_t>(desc->Sk, static_cast<int64_t>(desc->q_offset) + desc->Sq) : desc->Sk;
+    // a launch whose queries all see at least as many keys as they are themselves (a rank's share of a ring, a dense
+    // block): the waves of a workgroup then do nearly equal work, and workgroups of eight waves, which share every
+    // staged tile among twice as many waves, pay even where the launch has few of them
+    const bool rectangular = !desc->causal || desc->q_offset >= desc->Sq;
     if (groups(256) >= PICO_FWD_NW8_MIN) rc = launch<PICO_FWD_CFG64>(p, s);
-    else if (groups(128) >= 512) rc = launch<64, 1, 4, 64>(p, s);
+    else if (groups(128) >= 512) {
+      // (measured at B8, 256 queries x 1024 keys of every head: 26.9 us with eight waves, 30.1 us with four)
+      if (rectangular && groups(256) >= 256) rc = launch<PICO_FWD_CFG64>(p, s);
+      else rc = launch<64, 1, 4, 64>(p, s);
+    }
     // few waves in all: two waves per 32 queries, 64 keys of every 128 each -- in workgroups of eight waves (128 queries)
-    // when those still cover the CUs and the keys a query sees span several staged tiles (one rank's share of configs[1]:
-    // 19.8 -> 16.9 us for rank 3 of 4; with 256 keys the smaller workgroups are 2 % faster)
-    else if (groups(128) >= 256 && visible_keys >= 512) rc = launch<64, 1, 8, 128, 2>(p, s);
+    // when those still cover the CUs and the launch is rectangular (one rank's share of configs[1]: 19.8 -> 16.9 us for
+    // rank 3 of 4; on a whole causal sequence, or with 256 keys, the smaller workgroups are a few percent faster)
+    else if (groups(128) >= 256 && rectangular && visible_keys >= 512) rc = launch<64, 1, 8, 128, 2>(p, s);
     else rc = launch<64, 1, 4, 128, PICO_FWD_KS>(p, s);
   } else {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;

@@ -130,11 +130,12 @@ def test_head_dim_128_large_launch_ragged_lengths(ops, device, Sq, Sk, q_offset,
     (4, 8, 777, 1203, 0, False),       # 8-wave kernels, dense, rectangular
     (2, 32, 1024, 1024, 0, True),      # half the batch: the 4-wave kernels without key split
     (2, 8, 1000, 1290, 290, True),     # 4-wave kernels, ragged, shifted diagonal, GQA
-    (1, 8, 1000, 1290, 290, True),     # key-split kernels on the same lengths (eight waves per workgroup)
-    (1, 8, 500, 800, 300, True),       # key-split kernels, four waves per workgroup (fewer workgroups still)
-    (4, 32, 256, 1024, 768, True),     # rank 3 of 4 at configs[1]: key split, eight waves
-    (4, 32, 256, 256, 0, True),        # rank 0 of 4: key split, four waves (few keys)
-    (1, 8, 640, 700, 0, False),        # key split, eight waves, dense
+    (1, 8, 1000, 1290, 290, True),     # key-split kernels (four waves per workgroup) on the same lengths
+    (1, 8, 500, 800, 300, True),       # key-split kernels, fewer workgroups still
+    (4, 32, 256, 1024, 768, True),     # rank 3 of 4 at configs[1]: rectangular, key split with eight waves per workgroup
+    (4, 32, 256, 256, 0, True),        # rank 0 of 4: key split, four waves (few keys, not rectangular)
+    (1, 8, 1024, 700, 0, False),       # dense: key split, eight waves
+    (8, 32, 256, 1024, 768, True),     # rectangular with 256 workgroups of 256 queries: the 8-wave kernels
 ])
 def test_head_dim_64_every_launch_size_class(ops, device, B, Hkv, Sq, Sk, q_offset, causal):
     """head_dim 64 at 32 query heads: the library picks 8-wave, 4-wave or key-split workgroups (of eight or four waves) by
