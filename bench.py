@@ -214,6 +214,78 @@ class RingBench:
         self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
 
 
+def ring_api_extra(torch, ops, rb, iters=20):
+    """The public API at configs[1]: ring_attention() (RingAttentionFunc, context_parallel.py:14-51) forward and
+    backward for the four virtual cp ranks -- every rank's own q / k / v chunk tensors (leaves that require gradients),
+    the ranks played in ascending order, one backward over all of them.  Autograd, the mailbox, the chunks' publishing
+    nodes and the fp32 -> bf16 hand-back of dk / dv are all inside the timed region.  Timed as replays of a HIP graph of
+    the whole step (what a captured training step pays) and as eager launches (bound by the host: Python + autograd
+    per call)."""
+    import picotron_amd.process_group_manager as pgm
+    from picotron_amd.context_parallel import context_parallel as cp
+    W, Sc = rb.W, rb.Sc
+    mgr = pgm.setup_process_group_manager(1, W, 1, 1)
+    leaves = [[t[:, :, r * Sc:(r + 1) * Sc].clone().requires_grad_() for t in (rb.q, rb.k, rb.v)] for r in range(W)]
+    dos = [rb.do[:, :, r * Sc:(r + 1) * Sc].clone() for r in range(W)]
+    total_flops = sum(rb.flops())
+
+    def step():
+        outs = []
+        for r in range(W):
+            mgr.set_cp_rank(r)
+            outs.append(cp.ring_attention(*leaves[r], rb.scale, True))
+        torch.autograd.backward(outs, dos)
+
+    def clear():
+        for ts in leaves:
+            for t in ts:
+                t.grad = None
+
+    res = {"what": "ring_attention() forward + backward over the 4 virtual ranks of configs[1] through autograd "
+                   "(one launch per rank and direction over the chunk list; PICO_RING_PER_STEP=1 gives the per-step shape)"}
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(3):
+                clear()
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        clear()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            step()
+        preheat(torch, graph.replay, 0.2)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(iters):
+            graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        ms = start.elapsed_time(stop) / iters
+        res["graph_replay"] = {"ms_per_step": round(ms, 4), "TFLOP/s": round(total_flops / (ms * 1e-3) / 1e12, 2),
+                               "frac_of_mfma_peak": round(total_flops / (ms * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+        del graph
+    except Exception as e:   # a capture that the autograd engine or the allocator refuses: report it, keep the eager figure
+        res["graph_replay"] = {"error": repr(e)[:200]}
+        torch.cuda.synchronize()
+    for _ in range(3):
+        clear()
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        clear()
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / iters
+    res["eager"] = {"ms_per_step": round(ms, 4), "TFLOP/s": round(total_flops / (ms * 1e-3) / 1e12, 2),
+                    "note": "host-bound: Python, autograd and ctypes per call"}
+    pgm.setup_process_group_manager(1, 1, 1, 1)
+    return res
+
+
 def seq_len_extra(torch, ops, iters=10):
     """The headline step (one causal forward + backward launch set over whole sequences, head_dim 64, 32 heads) at the
     same 4096 tokens but longer sequences: configs[1]'s launches are one generation of workgroups whose loads and stores
@@ -439,11 +511,35 @@ def long_context_extra(torch, ops, iters=10):
     res = {"flops": flops, "one_launch_per_direction": {"ms": round(ms_f, 3), "TFLOP/s": round(flops / (ms_f * 1e-3) / 1e12, 1)},
            "one_launch_per_ring_step": {"ms": round(ms_r, 3), "TFLOP/s": round(flops / (ms_r * 1e-3) / 1e12, 1)}}
 
-    # RoPE at the rank's absolute positions (r * Sc + arange(Sc)): the q chunk and one K chunk, tables of the whole
-    # sequence, pos_offset instead of sliced tables
+    # The rank's step as the ring runs it, RoPE included ("RoPE applied with absolute position ids offset by chunk
+    # index"): K / V are the eight chunk tensors of the ranks (separate allocations; ranks 0..6 arrive rotated), rank 7
+    # rotates its own k chunk (one launch), q is rotated inside the forward at positions 7 * 4096 + row, and the
+    # backward un-rotates dq and dk of every chunk in its epilogues; dq in bf16, dk / dv of the chunks in fp32 (the
+    # ring's travelling accumulators).  One launch per direction over the chunk list.
     from picotron_amd.model import get_cos_sin
     cos, sin = get_cos_sin(W * Sc, D, 10000.0)
     cos, sin = cos.cuda(), sin.cuda()
+    k_raw = [k[:, :, c * Sc:(c + 1) * Sc].clone() for c in range(W)]
+    v_ch = [v[:, :, c * Sc:(c + 1) * Sc].clone() for c in range(W)]
+    k_rot = [ops.rope(k_raw[c], cos, sin, pos_offset=c * Sc) for c in range(W)]
+    dk_ch = [torch.empty(1, Hkv, Sc, D, dtype=torch.float32, device="cuda") for _ in range(W)]
+    dv_ch = [torch.empty(1, Hkv, Sc, D, dtype=torch.float32, device="cuda") for _ in range(W)]
+
+    def with_rope():
+        ops.rope(k_raw[r], cos, sin, pos_offset=r * Sc, out=k_rot[r])
+        o, l, q_rot = ops.attn_fwd_chunks(q, k_rot, v_ch, scale, True, r * Sc, rope=(cos, sin), q_pos_offset=r * Sc, want_q_rot=True)
+        ops.attn_bwd_chunks(do, q_rot, k_rot, v_ch, l, scale, True, r * Sc, dq, dk_ch, dv_ch, out=o, rope=(cos, sin),
+                            q_pos_offset=r * Sc, k_pos_offset=0)
+
+    ms_w, _ = graph_time(torch, with_rope, iters)
+    res["one_launch_per_direction_rope_inside_chunk_list"] = {
+        "ms": round(ms_w, 3), "TFLOP/s": round(flops / (ms_w * 1e-3) / 1e12, 1),
+        "note": "k of the rank's own chunk rotated by one launch, q inside the forward, dq / dk un-rotated inside the backward; "
+                "K / V as 8 separate chunk tensors, dk / dv per chunk in fp32"}
+    del k_raw, v_ch, k_rot, dk_ch, dv_ch
+
+    # RoPE at the rank's absolute positions (r * Sc + arange(Sc)): the q chunk and one K chunk, tables of the whole
+    # sequence, pos_offset instead of sliced tables
     q_rot = torch.empty_like(q)
     k_rot = torch.empty_like(k[:, :, :Sc])
     ms_q, _ = graph_time(torch, lambda: ops.rope(q, cos, sin, pos_offset=r * Sc, out=q_rot), 20, per_graph=10)
@@ -659,6 +755,7 @@ def main():
                                       "flops": r3_flops,
                                       "frac_of_mfma_peak": round(r3_flops / (ms_r3 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
                                       "schedule": "the last rank's share alone: 256 queries of every head over chunks 0..3"}
+        extras["ring_attention_api"] = ring_api_extra(torch, ops, rb)
         ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
         extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4),
                                               "frac_of_mfma_peak": round(total_flops / (ms_ring * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),

@@ -177,15 +177,17 @@ typedef struct pico_rope_tables {
   int32_t rows;
 } pico_rope_tables;
 
-/* replaces: apply_rotary_pos_emb on q (model.py:131 / :136) followed by the attention forward (model.py:154-157),
- * one chunk: q arrives UN-rotated and every query is rotated once, in the prologue of the workgroup that owns it
+/* replaces: apply_rotary_pos_emb on q (model.py:131 / :136) followed by the attention forward (model.py:154-157):
+ * q arrives UN-rotated and every query is rotated once, in the prologue of the workgroup that owns it
  * (position = q_pos_offset + row; fp32 arithmetic, one rounding, as pico_rope); k_rot must already be rotated
  * (pico_rope on k: a key tile is read by many workgroups, rotating it there would repeat the work).  If q_rot is
- * given the rotated q is written there (bf16, its own b/h/s strides, unit D stride) for pico_attn_bwd_rope.
- * Everything else as pico_attn_fwd with merge = 0.
+ * given the rotated q is written there (bf16, its own b/h/s strides with rows that do not overlap, unit D stride)
+ * for pico_attn_bwd_rope.  merge as in pico_attn_fwd: with merge = 1 the call is one step of a ring whose queries
+ * sit at positions q_pos_offset .. (update_rope_for_context_parallel, context_parallel.py:189-195, as an offset).
+ * Everything else as pico_attn_fwd.
  */
 int pico_attn_fwd_rope(const pico_attn_desc* desc, const void* q, const void* k_rot, const void* v, void* out,
-                       float* lse, int out_dtype, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
+                       float* lse, int out_dtype, int merge, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
                        const int64_t* q_rot_stride, void* stream);
 
 /* replaces: D = sum(dO * O, dim=-1)  context_parallel.py:145.
@@ -226,18 +228,63 @@ int pico_attn_bwd_fused(const pico_attn_desc* desc, const void* q, const void* k
                         void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
                         void* stream);
 
-/* replaces: the backward of "rotate q and k, then attend" (autograd of model.py:131-137 + :154-157) for one chunk:
+/* replaces: the backward of "rotate q and k, then attend" (autograd of model.py:131-137 + :154-157):
  * pico_attn_bwd_fused on the ROTATED q and k (q_rot as written by pico_attn_fwd_rope, k_rot from pico_rope), with the
  * backward of RoPE -- the rotation by the negative angle -- applied to dq and dk in the kernels' epilogues, in fp32,
- * before their one rounding.  dq and dk are therefore gradients w.r.t. the UN-rotated q and k; no separate RoPE pass
- * runs in the backward.  `out` is the bf16 forward output, `delta` an output as in pico_attn_bwd_fused; dq, dk and dv
- * are all required and are written (not accumulated).  Positions: q_pos_offset + query row, k_pos_offset + key row.
+ * before their one rounding (or before they are added to an fp32 accumulator: the rotation is linear).  dq and dk are
+ * therefore gradients w.r.t. the UN-rotated q and k; no separate RoPE pass runs in the backward.  `out` is the bf16
+ * forward output, `delta` an output as in pico_attn_bwd_fused; dq, dk and dv are all required.  dq_accumulate /
+ * dkv_accumulate as in pico_attn_bwd (one block of a ring adds to the rank's running dq and to the chunk's travelling
+ * dk / dv, context_parallel.py:85-106).  Positions: q_pos_offset + query row, k_pos_offset + key row (a ring block of
+ * rank r over chunk c: r * Sc and c * Sc).
  */
 int pico_attn_bwd_rope(const pico_attn_desc* desc, const void* q_rot, const void* k_rot, const void* v,
                        const void* dout, const void* out, const float* lse, float* delta,
-                       void* dq, const int64_t* dq_stride, int dq_dtype,
-                       void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
+                       void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate,
+                       void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
                        const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset, void* stream);
+
+/* ------------------------------------------------------------------ all ring steps of one rank in one launch
+ * replaces: the loops of RingAttentionFunc.forward / backward  context_parallel.py:30-45, :63-106  when the K / V
+ *           chunks a rank would receive step by step are all in this GPU's memory already (virtual ranks).
+ * K / V are `count` chunks of chunk_len keys each, given by their base pointers; every chunk is addressed with the
+ * descriptor's k_stride / v_stride (and dkv_stride), desc->Sk must equal count * chunk_len, and with count > 1
+ * chunk_len must be a multiple of 128 (otherwise PICO_ERR_SHAPE: run the ring step by step with pico_attn_fwd(merge)
+ * / pico_attn_bwd(accumulate)).  Key j of the launch is row j % chunk_len of chunk j / chunk_len and sits at position
+ * j: list the chunks in the order of their positions (for a causal ring: the chunks of ranks 0 .. r, q_offset =
+ * r * chunk_len).  The online softmax runs across the chunks inside the kernel -- no per-step partial result, no
+ * merge pass, no fp32 running out.
+ * Backward: dk[c] / dv[c] receive chunk c's gradient; a NULL pair means that chunk's gradient is not wanted; bit c of
+ * accumulate_mask adds to what is there (fp32 only: the chunk's travelling accumulators).
+ */
+#define PICO_MAX_KV_CHUNKS 16
+typedef struct pico_kv_chunks {
+  int32_t count;                       /* 1 .. PICO_MAX_KV_CHUNKS */
+  int32_t chunk_len;
+  const void* k[PICO_MAX_KV_CHUNKS];
+  const void* v[PICO_MAX_KV_CHUNKS];
+  void* dk[PICO_MAX_KV_CHUNKS];        /* backward only */
+  void* dv[PICO_MAX_KV_CHUNKS];
+  uint32_t accumulate_mask;
+  uint32_t reserved;
+} pico_kv_chunks;
+
+/* pico_attn_fwd over a chunk list.  rope = NULL: q and the chunks' k are used as they are.  rope != NULL: q is rotated
+ * in the kernel as in pico_attn_fwd_rope (position q_pos_offset + row; the chunks' k must be rotated already) and
+ * written to q_rot if that is given. */
+int pico_attn_fwd_chunks(const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, void* out, float* lse,
+                         int out_dtype, int merge, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
+                         const int64_t* q_rot_stride, void* stream);
+
+/* pico_attn_bwd_fused over a chunk list.  `out` (forward output, dtype out_dtype, addressed like dout) may be NULL:
+ * `delta` is then an input, otherwise it is written (by the dQ kernel's prologue when out is bf16 and dq is wanted, by
+ * an internal pre-pass otherwise).  dq NULL: not wanted.  rope != NULL: q and the chunks' k are the rotated tensors and
+ * dq / dk leave un-rotated as in pico_attn_bwd_rope (key position = k_pos_offset + key index of the launch). */
+int pico_attn_bwd_chunks(const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, const void* dout,
+                         const void* out, int out_dtype, const float* lse, float* delta,
+                         void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate,
+                         const int64_t* dkv_stride, int dkv_dtype,
+                         const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset, void* stream);
 
 /* fp32 -> bf16/fp32 conversion with layout change: src [B,H,S,D] contiguous fp32,
  * dst addressed by dst_stride (b,h,s).  Used to hand dq_acc back in the dtype / layout of q.

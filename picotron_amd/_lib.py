@@ -29,6 +29,16 @@ class RopeTables(Structure):
     _fields_ = [("cos", c_void_p), ("sin", c_void_p), ("pitch", c_int64), ("dtype", c_int32), ("rows", c_int32)]
 
 
+MAX_KV_CHUNKS = 16
+
+
+class KvChunks(Structure):
+    """Mirror of ``pico_kv_chunks``."""
+    _fields_ = [("count", c_int32), ("chunk_len", c_int32), ("k", c_void_p * MAX_KV_CHUNKS), ("v", c_void_p * MAX_KV_CHUNKS),
+                ("dk", c_void_p * MAX_KV_CHUNKS), ("dv", c_void_p * MAX_KV_CHUNKS), ("accumulate_mask", ctypes.c_uint32),
+                ("reserved", ctypes.c_uint32)]
+
+
 _P = c_void_p
 _I64 = c_int64
 SIGNATURES = {
@@ -44,9 +54,13 @@ SIGNATURES = {
     "pico_swiglu_bwd": (c_int, [_P] * 5 + [_I64] * 7 + [c_int, _P]),
     "pico_lse_merge": (c_int, [_P, _P, _P, _P, _I64, _I64, c_int, _P]),
     "pico_attn_fwd": (c_int, [POINTER(AttnDesc), _P, _P, _P, _P, _P, c_int, c_int, _P]),
-    "pico_attn_fwd_rope": (c_int, [POINTER(AttnDesc), _P, _P, _P, _P, _P, c_int, POINTER(RopeTables), c_int, _P, POINTER(c_int64), _P]),
-    "pico_attn_bwd_rope": (c_int, [POINTER(AttnDesc)] + [_P] * 5 + [_P, _P] + [_P, POINTER(c_int64), c_int, _P, _P, POINTER(c_int64), c_int,
+    "pico_attn_fwd_rope": (c_int, [POINTER(AttnDesc), _P, _P, _P, _P, _P, c_int, c_int, POINTER(RopeTables), c_int, _P, POINTER(c_int64), _P]),
+    "pico_attn_bwd_rope": (c_int, [POINTER(AttnDesc)] + [_P] * 5 + [_P, _P] + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int,
                                    POINTER(RopeTables), c_int, c_int, _P]),
+    "pico_attn_fwd_chunks": (c_int, [POINTER(AttnDesc), _P, POINTER(KvChunks), _P, _P, c_int, c_int, POINTER(RopeTables), c_int, _P,
+                                     POINTER(c_int64), _P]),
+    "pico_attn_bwd_chunks": (c_int, [POINTER(AttnDesc), _P, POINTER(KvChunks), _P, _P, c_int, _P, _P, _P, POINTER(c_int64), c_int, c_int,
+                                     POINTER(c_int64), c_int, POINTER(RopeTables), c_int, c_int, _P]),
     "pico_attn_bwd_preprocess": (c_int, [POINTER(AttnDesc), _P, _P, c_int, _P, _P, _P]),
     "pico_attn_bwd": (c_int, [POINTER(AttnDesc)] + [_P] * 6 + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int, _P]),
     "pico_attn_bwd_fused": (c_int, [POINTER(AttnDesc)] + [_P] * 5 + [c_int, _P, _P] + [_P, POINTER(c_int64), c_int, c_int, _P, _P, POINTER(c_int64), c_int, c_int, _P]),

@@ -51,7 +51,8 @@ class ContextCommunicate:
         self._slot = slot
 
     def send_recv(self, tensor_to_send, recv_tensor=None):
-        result = torch.zeros_like(tensor_to_send) if recv_tensor is None else recv_tensor
+        # (the receive buffer needs no clearing: wait() overwrites all of it, with the peer's chunk or with NaN)
+        result = torch.empty_like(tensor_to_send) if recv_tensor is None else recv_tensor
         self._pending.append((tensor_to_send, result))
         return result
 

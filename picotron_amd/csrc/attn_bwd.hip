@@ -30,10 +30,11 @@ struct BwdParams {
   const __bf16* out;   // fused-delta mode of the dQ kernel: the forward output, addressed like dout
   float* delta_w;      //   ... and where that kernel writes delta = sum_d dO * O for the dK/dV kernel
   void* dq;
-  void* dk;
-  void* dv;
+  void* dk[kMaxChunks];      // per K / V chunk; nullptr: that chunk's gradient is not wanted
+  void* dv[kMaxChunks];
+  uint32_t dkv_accumulate;   // bit c: chunk c's dk / dv are added to (fp32)
   int dq_f32, dq_accumulate;
-  int dkv_f32, dkv_accumulate;
+  int dkv_f32;
   int pair_ktiles;  // dK/dV kernel: a workgroup takes key tile t and then tile n-1-t (equal work under a causal mask)
   int64_t dqs[3];  // element strides (b, h, s) of dq
   int64_t dks[3];  // element strides (b, h, s) of dk and dv
@@ -41,67 +42,14 @@ struct BwdParams {
 };
 
 // =====================================================================================  dK / dV
-// bf16 gradients leave with streaming (non-temporal) stores unless built with -DPICO_STREAM_GRADS=0
-#ifndef PICO_STREAM_GRADS
-#define PICO_STREAM_GRADS 1
-#endif
-constexpr bool kStreamGrads = PICO_STREAM_GRADS != 0;
-#ifndef PICO_PIPELINE_TRIP
-#define PICO_PIPELINE_TRIP 1
-#endif
-constexpr bool kPipelineTrip = PICO_PIPELINE_TRIP != 0;
-#ifndef PICO_DKDV_STAGES128
-#define PICO_DKDV_STAGES128 1
-#endif
-#ifndef PICO_DKDV_STAGES64
-#define PICO_DKDV_STAGES64 1
-#endif
-// Layout of the Q / dO tiles in LDS (elements of padding per row, elements of skew after every 4 rows): see KvCfg
-#ifndef PICO_DKDV_LDQPAD
-#define PICO_DKDV_LDQPAD 32
-#endif
-#ifndef PICO_DKDV_SKEW
-#define PICO_DKDV_SKEW 8
-#endif
-// Wave priority in the two middle stages of a dK/dV trip (those that mix MFMAs with softmax arithmetic): raised, so
-// that of the two waves of a SIMD the one with vector work to hide issues first (-1.5 % at head_dim 64)
-#ifndef PICO_DKDV_PRIO
-#define PICO_DKDV_PRIO 1
-#endif
-// The scores are needed as exp2(s * sm_scale * log2e - lse * log2e).  With PICO_PRESCALE the factor is folded into one
-// bf16 operand of the S product once per kernel (K fragments in the dK/dV kernel, Q fragments in the dQ kernel) and
-// -lse * log2e is what the S accumulator starts from, so the exponent comes out of the MFMA and the multiply-add in
-// front of every v_exp_f32 disappears (one of about seven vector instructions per score).  The scaled operand is
-// rounded to bf16 once more: an error of 2^-9 relative per element, i.e. of the size of the inputs' own rounding.
-#ifndef PICO_PAIR_KREGS
-#define PICO_PAIR_KREGS 4
-#endif
-#ifndef PICO_PAIR_STAGE_TOP
-#define PICO_PAIR_STAGE_TOP 1
-#endif
-#ifndef PICO_PAIR_AHEAD
-#define PICO_PAIR_AHEAD 1
-#endif
-#ifndef PICO_PAIR_AHEAD_T
-#define PICO_PAIR_AHEAD_T 2
-#endif
-#ifndef PICO_PRESCALE
-#define PICO_PRESCALE 1
-#endif
-constexpr bool kPrescale = PICO_PRESCALE != 0;
-
-template <int N>
-__device__ __forceinline__ void scale_fragments(bf16x8 (&f)[N], float c) {
-#pragma unroll
-  for (int s = 0; s < N; ++s)
-#pragma unroll
-    for (int e = 0; e < 8; ++e) f[s][e] = static_cast<__bf16>(static_cast<float>(f[s][e]) * c);
-}
-
+// bf16 gradients leave with streaming (non-temporal) stores: nothing on this GPU reads them back soon
+constexpr bool kStreamGrads = true;
 // PAIR: eight waves instead of four; waves w and w + 4 (they share a SIMD) own the same 32 keys and split every
 // 64-query tile between them, one 32-query sub-block each, with accumulators of their own that are added through LDS
 // at the end of the key tile.  A wave then holds one sub-block's S / dP tiles instead of two, which is what lets the
 // head_dim 128 kernel fit 256 registers, i.e. two waves per SIMD.
+constexpr int kPairKRegs = 4;   // PAIR: K fragments (of D / 16) that stay in registers; the others are read from LDS
+
 template <int D, bool PAIR = false>
 struct KvCfg {
   static constexpr int NW = PAIR ? 8 : 4;
@@ -116,8 +64,8 @@ struct KvCfg {
   // pieces of 4 consecutive rows tile the banks (transposed reads at their minimum of 2 requests per bank; at a pitch
   // of D + 8 they take 3-4), and the 4-word skew per 4 rows spreads 16 consecutive rows over all multiples of 4 words
   // (row reads at their minimum of 4).
-  static constexpr int LDQ = D + PICO_DKDV_LDQPAD;
-  static constexpr int kSkew = PICO_DKDV_SKEW;
+  static constexpr int LDQ = D + 32;
+  static constexpr int kSkew = 8;
   static constexpr int kTileElems = BM * LDQ + kSkew * (BM / 4);       // one tile
   static constexpr int kTrStep = 8 * LDQ + 2 * kSkew;                  // 8 rows further down
   static constexpr int kVecPerRow = D / 8;
@@ -145,7 +93,10 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   const AttnParams& a = p.a;
   const int hkv = blockIdx.x % a.Hkv, b = blockIdx.x / a.Hkv;
   const int group = a.Hq / a.Hkv;
-  const int key0 = ktile * BN;
+  const int key0 = ktile * BN;                     // position of the tile's first key in the launch
+  const int chunk = a.kv.count > 1 ? key0 / a.kv.len : 0;
+  const int crow0 = key0 - chunk * a.kv.len;       // ... and its row in the chunk that holds it
+  if (p.dk[chunk] == nullptr) return;              // this chunk's gradient is not wanted (uniform over the workgroup)
   const int tid = threadIdx.x, wave_id = tid / 64, lane = tid % 64;
   // wave: which 32 keys of the tile; pair_sb (PAIR only): which 32-query sub-block of every query tile
   const int wave = PAIR ? __builtin_amdgcn_readfirstlane(wave_id % C::kKeyWaves) : wave_id;
@@ -153,8 +104,8 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   const int n = lane % 32, h = lane / 32;
   const float c = a.sm_scale * kLog2e;
 
-  const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
-  const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
+  const __bf16* kbase = a.kv.k[chunk] + b * a.ks[0] + hkv * a.ks[1];
+  const __bf16* vbase = a.kv.v[chunk] + b * a.vs[0] + hkv * a.vs[1];
 
   // ---- K, V fragments of this wave's 32 keys (B operand: lane = key, 8 consecutive d per k step), fetched
   //      row-major and turned into fragments through the wave's piece of the SECOND tile buffer, which nothing
@@ -169,9 +120,9 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   if (loads_kv) {
     // (the wave index read as a scalar: the buffer windows below are then built in scalar registers; from the
     // per-lane value the compiler cannot tell that they are the same in all lanes and loops over the lanes' values)
-    const int row0 = key0 + 32 * __builtin_amdgcn_readfirstlane(wave);
-    kt.issue(make_buffer(kbase + static_cast<int64_t>(row0) * a.ks[2], span_bytes(a.Sk - row0, a.ks[2], D)), a.ks[2], lane);
-    vt.issue(make_buffer(vbase + static_cast<int64_t>(row0) * a.vs[2], span_bytes(a.Sk - row0, a.vs[2], D)), a.vs[2], lane);
+    const int row0 = crow0 + 32 * __builtin_amdgcn_readfirstlane(wave);
+    kt.issue(make_buffer(kbase + static_cast<int64_t>(row0) * a.ks[2], span_bytes(a.kv.len - row0, a.ks[2], D)), a.ks[2], lane);
+    vt.issue(make_buffer(vbase + static_cast<int64_t>(row0) * a.vs[2], span_bytes(a.kv.len - row0, a.vs[2], D)), a.vs[2], lane);
   }
 
   f32x16 dk_acc[D / 32], dv_acc[D / 32];
@@ -262,8 +213,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     if (tid < BM) {
       // rows past Sq, and rows whose lse is -inf (they saw no key), get lse = +inf so that P = 0
       const bool live = static_cast<uint32_t>(tid) * 4u < cur.rows_left && lreg != -INFINITY;
-      // (with kPrescale the value is the S accumulator's start, so it is stored negated)
-      sL[tid] = kPrescale ? (live ? -lreg * kLog2e : -INFINITY) : (live ? lreg * kLog2e : INFINITY);
+      sL[tid] = live ? lreg * kLog2e : INFINITY;
       sDelta[tid] = -dreg;   // stored negated: it is loaded straight into the dP accumulator (0 past Sq)
     }
   };
@@ -277,15 +227,9 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       unsigned char* region = smem_raw + C::kBufBytes + wave * WaveTile<D>::kRegionBytes;
       kt.fragments(region, lane, kf);
       vt.fragments(region, lane, vf);
-      if constexpr (kPrescale) scale_fragments(kf, c);   // kf feeds the S product only (dK comes from Q^T dS)
     } else {
-      // the first wave of each pair leaves both tiles in the pair's piece of LDS, K with the scale folded in
+      // the first wave of each pair leaves both tiles in the pair's piece of LDS
       kt.fragments(pair_k, lane, kf);
-      if constexpr (kPrescale) {
-        scale_fragments(kf, c);
-#pragma unroll
-        for (int s = 0; s < D / 16; ++s) *reinterpret_cast<bf16x8*>(pair_k + n * kFragPitch + (16 * s + 8 * h) * 2) = kf[s];
-      }
       vt.fragments(pair_v, lane, vf);
     }
   }
@@ -293,7 +237,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     __syncthreads();
     // the first few K fragments stay in registers (as many as fit beside the accumulators)
 #pragma unroll
-    for (int j = 0; j < PICO_PAIR_KREGS; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
+    for (int j = 0; j < kPairKRegs; ++j) kf[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
   }
   if (n_iter > 0) stage(0);
   // The K / V fragment loads above are complete by now on every path that enters the loop (the LDS fill
@@ -302,11 +246,11 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   // of the NEXT tile on every trip.
   __builtin_amdgcn_s_waitcnt(kWaitVmcnt0);
   __syncthreads();
-  // PAIR (PICO_PAIR_STAGE_TOP): the tile after the one being computed goes to LDS at the TOP of a trip, from loads that
+  // PAIR: the tile after the one being computed goes to LDS at the TOP of a trip, from loads that
   // were issued at the top of the trip before; the registers are then reloaded with the tile after that.  The LDS
   // writes are off the end of the trip (where every wave of the workgroup would wait for them in front of the barrier)
   // and a load has a whole trip to arrive.
-  constexpr bool kStageTop = PAIR && PICO_PAIR_STAGE_TOP != 0;
+  constexpr bool kStageTop = PAIR;
   if constexpr (kStageTop) {
     if (n_iter > 1) { advance(); prefetch(); }
   }
@@ -339,20 +283,18 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 * sb + 8 * j + 4 * h]);
-        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (kPrescale) s4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
-        for (int t = 0; t < 4; ++t) { s_acc[4 * j + t] = s4[t]; dp_acc[4 * j + t] = d4[t]; }
+        for (int t = 0; t < 4; ++t) { s_acc[4 * j + t] = 0.f; dp_acc[4 * j + t] = d4[t]; }
       }
       if constexpr (PAIR) {
         // both operands of every MFMA come from LDS: they are requested kAhead steps before the MFMAs that use them, and
         // the scheduling barriers keep that order (left alone, the compiler reuses one set of registers and every MFMA
         // waits for an LDS round trip)
-        constexpr int kSteps = D / 16, kAhead = PICO_PAIR_AHEAD;
+        constexpr int kSteps = D / 16, kAhead = 1;
         bf16x8 qa[kSteps], da[kSteps], kb[kSteps], vb[kSteps];
         auto fetch = [&](int j) {
           qa[j] = *reinterpret_cast<const bf16x8*>(&sQ[tile_row(32 * sb + n) + 16 * j + 8 * h]);
-          if (j >= PICO_PAIR_KREGS) kb[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
+          if (j >= kPairKRegs) kb[j] = *reinterpret_cast<const bf16x8*>(pair_k + n * kFragPitch + (16 * j + 8 * h) * 2);
           da[j] = *reinterpret_cast<const bf16x8*>(&sdO[tile_row(32 * sb + n) + 16 * j + 8 * h]);
           vb[j] = *reinterpret_cast<const bf16x8*>(pair_v + n * kFragPitch + (16 * j + 8 * h) * 2);
         };
@@ -362,7 +304,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
 #pragma unroll
         for (int j = 0; j < kSteps; ++j) {
           if (j + kAhead < kSteps) fetch(j + kAhead);
-          s_acc = mfma32(qa[j], j < PICO_PAIR_KREGS ? kf[j] : kb[j], s_acc);
+          s_acc = mfma32(qa[j], j < kPairKRegs ? kf[j] : kb[j], s_acc);
           dp_acc = mfma32(da[j], vb[j], dp_acc);
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -384,12 +326,11 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       const int key_rel = kw0 + n - qs_pos - 4 * h;  // key is masked for row (8j + 4h + t) iff key_rel > 8j + t
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        f32x4 l4 = {0.f, 0.f, 0.f, 0.f};
-        if constexpr (!kPrescale) l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[32 * sb + 8 * j + 4 * h]);
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const int i = 4 * j + t;
-          float pv = kPrescale ? fast_exp2(s_acc[i]) : fast_exp2(s_acc[i] * c - l4[t]);
+          float pv = fast_exp2(s_acc[i] * c - l4[t]);
           if constexpr (kMask) {
             if (key_rel > 8 * j + t) pv = 0.f;
           }
@@ -403,7 +344,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     // dO^T / Q^T from the row-major LDS tiles through transposing reads.
     auto accumulate = [&](int sb, const f32x16& s_acc, const f32x16& dp_acc) {
       if constexpr (PAIR) {
-        constexpr int kSlots = 2 * (D / 32), kAhead = PICO_PAIR_AHEAD_T;
+        constexpr int kSlots = 2 * (D / 32), kAhead = 2;
         bf16x8 dof[kSlots], qf[kSlots];
         auto fetch = [&](int idx) {
           const int cc = idx / (D / 32), db = idx % (D / 32);
@@ -444,14 +385,13 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
     };
 
-    const bool off_diagonal = !PAIR && kPipelineTrip && BM == 64 && (!a.causal || kw0 + 31 <= a.q_offset + q0);
+    const bool off_diagonal = !PAIR && (!a.causal || kw0 + 31 <= a.q_offset + q0);
     if (!kStageTop && has_next && !off_diagonal) prefetch();
     if (off_diagonal) {
       // Every pair of this trip is visible to this wave (all trips off the diagonal): straight-line code in an order
       // that lets the wave's own phases overlap -- the matrix pipe works on the second sub-block's S / dP while the
       // vector pipe does the first one's softmax, and on the first one's dV / dK during the second one's softmax.
       f32x16 s0, d0, s1, d1;
-      if constexpr (D >= 128 ? PICO_DKDV_STAGES128 != 0 : PICO_DKDV_STAGES64 != 0) {
       // Four stages; in the middle two, every pair of MFMAs is followed in program order by a share of the OTHER
       // sub-block's softmax arithmetic and by the LDS reads of a later pair.  A wave issues in order: vector
       // instructions that merely follow a batch of MFMAs start when the batch has been issued, i.e. when the matrix
@@ -466,7 +406,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       auto softmax_part = [&](f32x16& s_acc, f32x16& dp_acc, const f32x4 (&l4)[4], int first, int count) {
 #pragma unroll
         for (int i = first; i < first + count; ++i) {
-          const float pv = kPrescale ? fast_exp2(s_acc[i]) : fast_exp2(s_acc[i] * c - l4[i / 4][i % 4]);
+          const float pv = fast_exp2(s_acc[i] * c - l4[i / 4][i % 4]);
           s_acc[i] = pv;
           dp_acc[i] = pv * dp_acc[i];
         }
@@ -474,23 +414,21 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       // stage A: products of sub-block 0
       products(0, s0, d0);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (PICO_DKDV_PRIO != 0) __builtin_amdgcn_s_setprio(PICO_DKDV_PRIO);
+      __builtin_amdgcn_s_setprio(1);
       // stage B: products of sub-block 1, softmax of sub-block 0 between them
       {
         // lse rows of sub-block 0 are fetched a slot ahead of the elements that need them (kPer elements per slot)
         constexpr int kPer = 16 / kPairs;
         f32x4 l4[4];
         auto lse_row = [&](int r) {
-          if constexpr (!kPrescale) l4[r] = *reinterpret_cast<const f32x4*>(&sL[8 * r + 4 * h]);
+          l4[r] = *reinterpret_cast<const f32x4*>(&sL[8 * r + 4 * h]);
         };
         lse_row(0);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sDelta[32 + 8 * j + 4 * h]);
-          f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
-          if constexpr (kPrescale) s4 = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * j + 4 * h]);
 #pragma unroll
-          for (int t = 0; t < 4; ++t) { s1[4 * j + t] = s4[t]; d1[4 * j + t] = d4[t]; }
+          for (int t = 0; t < 4; ++t) { s1[4 * j + t] = 0.f; d1[4 * j + t] = d4[t]; }
         }
         bf16x8 qa[kPairs], da[kPairs];
         auto fetch = [&](int j) {
@@ -516,7 +454,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
         constexpr int kPer = 16 / kSlots;
         f32x4 l4[4];
         auto lse_row = [&](int r) {
-          if constexpr (!kPrescale) l4[r] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * r + 4 * h]);
+          l4[r] = *reinterpret_cast<const f32x4*>(&sL[32 + 8 * r + 4 * h]);
         };
         lse_row(0);
         bf16x8 dof[kSlots], qf[kSlots];
@@ -544,20 +482,9 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
       }
       // stage D: dV / dK of sub-block 1; the next tile's global loads are issued here, not at the top of the trip:
       // their registers are free until now
-      if constexpr (PICO_DKDV_PRIO != 0) __builtin_amdgcn_s_setprio(0);
+      __builtin_amdgcn_s_setprio(0);
       if (has_next) prefetch();
       accumulate(1, s1, d1);
-      } else {
-      products(0, s0, d0);
-      products(1, s1, d1);
-      __builtin_amdgcn_sched_barrier(0);
-      softmax_grad(0, s0, d0, std::false_type{});
-      accumulate(0, s0, d0);
-      __builtin_amdgcn_sched_barrier(0);
-      if (has_next) prefetch();  // issued here, not at the top of the trip: its registers are free until now
-      softmax_grad(1, s1, d1, std::false_type{});
-      accumulate(1, s1, d1);
-      }
     } else {
 #pragma unroll
       for (int sbi = 0; sbi < (PAIR ? 1 : BM / 32); ++sbi) {
@@ -609,17 +536,18 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   }
   if (!PAIR || pair_sb == 0) {
     unsigned char* region = smem_raw + wave * kRowRegionBytes;
-    const int row0 = key0 + 32 * wave;
-    const int rows_live = a.Sk - row0;
+    const int row0 = crow0 + 32 * wave;          // first row of the wave inside its chunk
+    const int rows_live = a.kv.len - row0;
     const int64_t off = b * p.dks[0] + hkv * p.dks[1] + static_cast<int64_t>(row0) * p.dks[2];
-    // gradient w.r.t. the un-rotated k: rotate the lane's row of dK back (linear, so the scale can follow)
-    if (p.rope.cos != nullptr) rope_unrotate_acc<D>(dk_acc, p.rope, n < rows_live ? p.rope.k_pos0 + row0 + n : 0, h);
+    // gradient w.r.t. the un-rotated k: rotate the lane's row of dK back (linear, so the scale and the sum can follow)
+    if (p.rope.cos != nullptr) rope_unrotate_acc<D>(dk_acc, p.rope, n < rows_live ? p.rope.k_pos0 + kw0 + n : 0, h);
+    const bool accumulate = (p.dkv_accumulate >> chunk) & 1u;
     if (p.dkv_f32) {
-      wave_store_rows<D, true>(region, dk_acc, a.sm_scale, static_cast<float*>(p.dk) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
-      wave_store_rows<D, true>(region, dv_acc, 1.f, static_cast<float*>(p.dv) + off, p.dks[2], rows_live, lane, p.dkv_accumulate, false);
+      wave_store_rows<D, true>(region, dk_acc, a.sm_scale, static_cast<float*>(p.dk[chunk]) + off, p.dks[2], rows_live, lane, accumulate, false);
+      wave_store_rows<D, true>(region, dv_acc, 1.f, static_cast<float*>(p.dv[chunk]) + off, p.dks[2], rows_live, lane, accumulate, false);
     } else {
-      wave_store_rows<D, false>(region, dk_acc, a.sm_scale, static_cast<__bf16*>(p.dk) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
-      wave_store_rows<D, false>(region, dv_acc, 1.f, static_cast<__bf16*>(p.dv) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
+      wave_store_rows<D, false>(region, dk_acc, a.sm_scale, static_cast<__bf16*>(p.dk[chunk]) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
+      wave_store_rows<D, false>(region, dv_acc, 1.f, static_cast<__bf16*>(p.dv[chunk]) + off, p.dks[2], rows_live, lane, false, kStreamGrads);
     }
   }
 }
@@ -647,11 +575,9 @@ __device__ __forceinline__ void attn_bwd_dkdv_body(const BwdParams& p) {
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void attn_bwd_dkdv_kernel_d64(const BwdParams p) {
   attn_bwd_dkdv_body<64>(p);
 }
-#ifndef PICO_DKDV_PAIR128
-#define PICO_DKDV_PAIR128 1
-#endif
-__global__ __launch_bounds__(PICO_DKDV_PAIR128 ? 512 : 256) void attn_bwd_dkdv_kernel_d128(const BwdParams p) {
-  attn_bwd_dkdv_body<128, PICO_DKDV_PAIR128 != 0>(p);
+// D = 128: eight waves, two per key block (see KvCfg), 256 registers each
+__global__ __launch_bounds__(512) void attn_bwd_dkdv_kernel_d128(const BwdParams p) {
+  attn_bwd_dkdv_body<128, true>(p);
 }
 
 template <int D> struct KvKernel;
@@ -661,10 +587,6 @@ template <> struct KvKernel<128> { static constexpr auto fn = &attn_bwd_dkdv_ker
 // =====================================================================================  dQ
 // KS > 1: KS waves share the same 32 queries and each takes one 64-key step of every staged tile (see the forward
 // kernel); their dQ partial sums meet in LDS at the end.
-// workgroups of 256 queries (8 waves) a launch must have before that size is used
-#ifndef PICO_DQ_NW8_MIN
-#define PICO_DQ_NW8_MIN 512
-#endif
 template <int D, int NW, int KT, int KS = 1>
 struct DqCfg {
   static constexpr int kThreads = 64 * NW;
@@ -703,11 +625,6 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
   const int n = lane % 32, h = lane / 32;
   const int qw = wave % C::kQWaves, ks = wave / C::kQWaves;   // which queries, which 64-key step of a staged tile
   const float c = a.sm_scale * kLog2e;
-  // (at head_dim 128 the kernel has no registers left for the accumulator's 16-register start value)
-  constexpr bool kPre = kPrescale && D <= 64;
-
-  const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
-  const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
 
   // ---- per-lane query: Q and dO fragments (B operands: fetched row-major, turned into fragments through the
   //      wave's piece of LDS; the tile buffers are filled only after the barrier below), lse and delta
@@ -735,7 +652,6 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
     unsigned char* region = smem_raw + wave * WaveTile<D>::kRegionBytes;
     qt.fragments(region, lane, qf);
     dt.fragments(region, lane, dof);
-    if constexpr (kPre) scale_fragments(qf, c);   // qf feeds the S product only
     if constexpr (kDelta) {
       // delta = sum_d dO * O of the lane's row (context_parallel.py:145): each half of the wave holds half of the
       // row's columns in its fragments; the dK/dV kernel, launched after this one, reads the result from memory
@@ -778,20 +694,17 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
     k_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.ks[2] + cv * 8) * 2);
     v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
   }
-  // a cursor walks the key tiles in order: stepping it is four scalar adds instead of 64-bit multiplies
-  const char* k_ptr = reinterpret_cast<const char*>(kbase);
-  const char* v_ptr = reinterpret_cast<const char*>(vbase);
-  uint32_t k_left = span_bytes(a.Sk, a.ks[2], D), v_left = span_bytes(a.Sk, a.vs[2], D);
-  const uint32_t k_step = static_cast<uint32_t>(KT * a.ks[2] * 2), v_step = static_cast<uint32_t>(KT * a.vs[2] * 2);
+  // a cursor walks the key tiles in order (and from chunk to chunk): stepping it is a few scalar adds
+  KvCursor<D> cur;
+  cur.open(a, 0, b, hkv, KT);
   auto load_tile = [&]() {  // the next tile of KT keys
-    const buffer_rsrc kb = make_buffer(k_ptr, k_left), vb = make_buffer(v_ptr, v_left);
+    const buffer_rsrc kb = make_buffer(cur.k, cur.k_left), vb = make_buffer(cur.v, cur.v_left);
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       kreg[i] = buffer_load_b128(kb, k_off[i]);
       vreg[i] = buffer_load_b128(vb, v_off[i]);
     }
-    k_ptr += k_step;  k_left -= k_step;
-    v_ptr += v_step;  v_left -= v_step;
+    cur.next(a);
   };
   auto store_tile = [&](int buf) {
     __bf16* sK = smem + buf * C::kTileElems;
@@ -837,9 +750,9 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
       if constexpr (KS == 1) __builtin_amdgcn_iglp_opt(0);
 #pragma unroll
       for (int mb = 0; mb < BN / 32; ++mb) {
-        // dP - delta comes out of the MFMA, and with kPre so does the exponent s * c - lse * log2e
+        // dP - delta comes out of the MFMA
 #pragma unroll
-        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = kPre ? -lse2 : 0.f; dp_acc[mb][i] = -delta; }
+        for (int i = 0; i < 16; ++i) { s_acc[mb][i] = 0.f; dp_acc[mb][i] = -delta; }
 #pragma unroll
         for (int s = 0; s < D / 16; ++s) {
           const bf16x8 ka = *reinterpret_cast<const bf16x8*>(&sKs[(32 * mb + n) * LDK + 16 * s + 8 * h]);
@@ -866,7 +779,7 @@ __global__ __launch_bounds__(64 * NW, (NW <= 4 && D <= 64) ? 2 : 1) void attn_bw
       for (int mb = 0; mb < BN / 32; ++mb)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-          const float pv = kPre ? fast_exp2(s_acc[mb][i]) : fast_exp2(s_acc[mb][i] * c - lse2);
+          const float pv = fast_exp2(s_acc[mb][i] * c - lse2);
           dp_acc[mb][i] = pv * dp_acc[mb][i];
         }
       // ---- dQ^T[d][query] += K^T[d][key] dS^T[key][query]
@@ -969,7 +882,7 @@ __global__ __launch_bounds__(256) void attn_bwd_preprocess_kernel(const __bf16* 
 
 template <int D>
 int launch_dkdv(const BwdParams& p, hipStream_t s) {
-  using C = KvCfg<D, D == 128 && PICO_DKDV_PAIR128 != 0>;
+  using C = KvCfg<D, D == 128>;
   static LdsOnce lds_reserved;
   if (!reserve_lds_once(lds_reserved, reinterpret_cast<const void*>(KvKernel<D>::fn), C::kLdsBytes))
     return fail(PICO_ERR_LAUNCH, "pico_attn_bwd(dk/dv): cannot reserve %zu bytes of LDS", C::kLdsBytes);
@@ -1032,37 +945,50 @@ extern "C" int pico_attn_bwd_preprocess(const pico_attn_desc* desc, const void* 
 
 namespace {
 
-// Shared body of pico_attn_bwd and pico_attn_bwd_fused.  With `out` (bf16 forward output) the dQ kernel computes
-// delta itself, writes it to `delta_w`, and runs BEFORE the dK/dV kernel, which reads it from there.
-int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
+// Shared body of the backward entry points.  With `out` (bf16 forward output) the dQ kernel computes delta itself,
+// writes it to `delta_w`, and runs BEFORE the dK/dV kernel, which reads it from there.
+int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, const void* dout,
             const float* lse, const float* delta, const void* out, float* delta_w, void* dq, const int64_t* dq_stride,
-            int dq_dtype, int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
-            int dkv_accumulate, void* stream, const RopeArgs* rope = nullptr) {
+            int dq_dtype, int dq_accumulate, const int64_t* dkv_stride, int dkv_dtype, void* stream,
+            const RopeArgs* rope = nullptr) {
   if ((dkv_dtype != PICO_BF16 && dkv_dtype != PICO_F32) || (dq_dtype != PICO_BF16 && dq_dtype != PICO_F32))
     return fail(PICO_ERR_DTYPE, "%s: gradient dtype codes %d / %d not supported", fn, dq_dtype, dkv_dtype);
-  if ((dkv_accumulate && dkv_dtype != PICO_F32) || (dq_accumulate && dq_dtype != PICO_F32))
-    return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
-  if (desc->B == 0) return PICO_OK;
-  // a gradient that is not wanted is passed as NULL and its kernel is skipped
-  const bool want_dq = dq != nullptr, want_dkv = dk != nullptr || dv != nullptr;
-  if (want_dkv && (!dk || !dv)) return fail(PICO_ERR_NULL, "%s: dk and dv must be given together", fn);
-  const bool have_q = desc->Sq > 0 && want_dq, have_k = desc->Sk > 0 && want_dkv;
-  if (((have_q || have_k) && desc->Sq > 0 && (!q || !dout || !lse || !delta)) ||
-      ((have_q || have_k) && desc->Sk > 0 && (!k || !v)))
-    return fail(PICO_ERR_NULL, "%s: q, k, v, dout, lse and delta are required", fn);
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(dout) || !aligned16(dq) || !aligned16(dk) ||
-      !aligned16(dv) || !aligned16(out))
-    return fail(PICO_ERR_ALIGN, "%s: q, k, v, dout, out, dq, dk and dv must be 16-byte aligned", fn);
+  if (dq_accumulate && dq_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
   BwdParams p;
-  p.a = make_params(desc, q, k, v);
+  p.a = make_params(desc, q, nullptr, nullptr);
+  if (int rc = set_chunks(fn, desc, kv, p.a, false)) return rc;
+  if (desc->B == 0) return PICO_OK;
+  // a gradient that is not wanted is passed as NULL and its kernel (or its chunk's workgroups) is skipped
+  bool want_dkv = false;
+  p.dkv_accumulate = 0;
+  for (int c = 0; c < kMaxChunks; ++c) p.dk[c] = p.dv[c] = nullptr;
+  for (int c = 0; c < kv->count; ++c) {
+    if ((kv->dk[c] == nullptr) != (kv->dv[c] == nullptr))
+      return fail(PICO_ERR_NULL, "%s: dk and dv must be given together (chunk %d)", fn, c);
+    p.dk[c] = kv->dk[c];
+    p.dv[c] = kv->dv[c];
+    if (kv->dk[c]) {
+      want_dkv = true;
+      if ((kv->accumulate_mask >> c) & 1u) p.dkv_accumulate |= 1u << c;
+    }
+  }
+  if (p.dkv_accumulate && dkv_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
+  const bool want_dq = dq != nullptr;
+  const bool have_q = desc->Sq > 0 && want_dq, have_k = desc->Sk > 0 && want_dkv;
+  if ((have_q || have_k) && desc->Sq > 0 && (!q || !dout || !lse || !delta))
+    return fail(PICO_ERR_NULL, "%s: q, dout, lse and delta are required", fn);
+  if ((have_q || have_k) && desc->Sk > 0)
+    for (int c = 0; c < kv->count; ++c)
+      if (!kv->k[c] || !kv->v[c]) return fail(PICO_ERR_NULL, "%s: k / v of chunk %d are NULL", fn, c);
+  if (!aligned16(q) || !aligned16(dout) || !aligned16(dq) || !aligned16(out))
+    return fail(PICO_ERR_ALIGN, "%s: q, dout, out and dq must be 16-byte aligned", fn);
   p.dout = static_cast<const __bf16*>(dout);
-  p.lse = lse; p.delta = delta; p.dq = dq; p.dk = dk; p.dv = dv;
+  p.lse = lse; p.delta = delta; p.dq = dq;
   p.out = static_cast<const __bf16*>(out);
   p.delta_w = delta_w;
   p.dq_f32 = dq_dtype == PICO_F32;
   p.dq_accumulate = dq_accumulate != 0;
   p.dkv_f32 = dkv_dtype == PICO_F32;
-  p.dkv_accumulate = dkv_accumulate != 0;
   p.pair_ktiles = 0;
   p.rope = rope ? *rope : RopeArgs{nullptr, nullptr, 0, 0, 0, 0};
   auto strides = [&](const int64_t* given, int heads, int seq, int64_t (&st)[3], int align) -> bool {
@@ -1078,7 +1004,7 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
     }
     return true;
   };
-  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, p.dq_f32 ? 4 : 8) || !strides(dkv_stride, desc->Hkv, desc->Sk, p.dks, 8))
+  if (!strides(dq_stride, desc->Hq, desc->Sq, p.dqs, p.dq_f32 ? 4 : 8) || !strides(dkv_stride, desc->Hkv, kv->chunk_len, p.dks, 8))
     return fail(PICO_ERR_STRIDE, "%s: dq strides must be non-negative multiples of 4 (fp32) or 8 (bf16), dk/dv strides of 8", fn);
   hipStream_t s = static_cast<hipStream_t>(stream);
   auto run_dkdv = [&]() -> int {
@@ -1098,7 +1024,7 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
       // the forward's rules: eight waves per workgroup also for rectangular launches (every query sees at least as many
       // keys as there are queries) with fewer workgroups than the square ones need
       const bool rectangular = !desc->causal || desc->q_offset >= desc->Sq;
-      if (groups(256) >= PICO_DQ_NW8_MIN) rc = launch_dq<64, 8, 64>(p, s);
+      if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
       else if (groups(128) >= 512) {
         if (rectangular && groups(256) >= 256) rc = launch_dq<64, 8, 64>(p, s);
         else rc = launch_dq<64, 4, 64>(p, s);
@@ -1122,6 +1048,46 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
   return run_dq();
 }
 
+pico_kv_chunks one_chunk(const pico_attn_desc* desc, const void* k, const void* v, void* dk, void* dv, int accumulate) {
+  pico_kv_chunks kv = {};
+  kv.count = 1;
+  kv.chunk_len = desc->Sk;
+  kv.k[0] = k;
+  kv.v[0] = v;
+  kv.dk[0] = dk;
+  kv.dv[0] = dv;
+  kv.accumulate_mask = accumulate ? 1u : 0u;
+  return kv;
+}
+
+// delta inside the dQ kernel needs that kernel to run and a bf16 out; otherwise the pre-pass computes it
+int run_bwd_with_out(const char* fn, const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, const void* dout,
+                     const void* out, int out_dtype, const float* lse, float* delta, void* dq, const int64_t* dq_stride,
+                     int dq_dtype, int dq_accumulate, const int64_t* dkv_stride, int dkv_dtype, void* stream,
+                     const RopeArgs* rope) {
+  if (out_dtype != PICO_BF16 && out_dtype != PICO_F32)
+    return fail(PICO_ERR_DTYPE, "%s: out dtype code %d not supported", fn, out_dtype);
+  if (desc->B == 0) return PICO_OK;
+  if (desc->Sq > 0 && (!out || !delta)) return fail(PICO_ERR_NULL, "%s: out and delta are required", fn);
+  const bool in_kernel = out_dtype == PICO_BF16 && dq != nullptr && desc->Sq > 0;
+  if (!in_kernel) {
+    if (int rc = pico_attn_bwd_preprocess(desc, dout, out, out_dtype, delta, nullptr, stream)) return rc;
+    return run_bwd(fn, desc, q, kv, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype, dq_accumulate, dkv_stride,
+                   dkv_dtype, stream, rope);
+  }
+  return run_bwd(fn, desc, q, kv, dout, lse, delta, out, delta, dq, dq_stride, dq_dtype, dq_accumulate, dkv_stride, dkv_dtype,
+                 stream, rope);
+}
+
+int rope_args(const char* fn, const pico_attn_desc* desc, const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset,
+              RopeArgs& r) {
+  if (q_pos_offset < 0 || k_pos_offset < 0) return fail(PICO_ERR_SHAPE, "%s: position offsets must be >= 0", fn);
+  const int64_t last = std::max(static_cast<int64_t>(q_pos_offset) + desc->Sq, static_cast<int64_t>(k_pos_offset) + desc->Sk) - 1;
+  if (int rc = check_rope_tables(fn, rope, desc->D, last)) return rc;
+  r = RopeArgs{rope->cos, rope->sin, rope->pitch, rope->dtype == PICO_F32, q_pos_offset, k_pos_offset};
+  return PICO_OK;
+}
+
 }  // namespace
 
 extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, const void* dout,
@@ -1129,47 +1095,57 @@ extern "C" int pico_attn_bwd(const pico_attn_desc* desc, const void* q, const vo
                              int dq_accumulate, void* dk, void* dv, const int64_t* dkv_stride, int dkv_dtype,
                              int dkv_accumulate, void* stream) {
   if (int rc = check_attn_desc("pico_attn_bwd", desc)) return rc;
-  return run_bwd("pico_attn_bwd", desc, q, k, v, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype, dq_accumulate,
-                 dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
+  if (dkv_accumulate && dkv_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "pico_attn_bwd: accumulate needs fp32 gradients");
+  const pico_kv_chunks kv = one_chunk(desc, k, v, dk, dv, dkv_accumulate);
+  return run_bwd("pico_attn_bwd", desc, q, &kv, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype, dq_accumulate,
+                 dkv_stride, dkv_dtype, stream);
 }
 
 extern "C" int pico_attn_bwd_fused(const pico_attn_desc* desc, const void* q, const void* k, const void* v,
                                    const void* dout, const void* out, int out_dtype, const float* lse, float* delta,
                                    void* dq, const int64_t* dq_stride, int dq_dtype, int dq_accumulate, void* dk, void* dv,
                                    const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate, void* stream) {
-  if (int rc = check_attn_desc("pico_attn_bwd_fused", desc)) return rc;
-  if (out_dtype != PICO_BF16 && out_dtype != PICO_F32)
-    return fail(PICO_ERR_DTYPE, "pico_attn_bwd_fused: out dtype code %d not supported", out_dtype);
-  if (desc->B == 0) return PICO_OK;
-  if (desc->Sq > 0 && (!out || !delta)) return fail(PICO_ERR_NULL, "pico_attn_bwd_fused: out and delta are required");
-  // delta inside the dQ kernel needs that kernel to run and a bf16 out; otherwise the pre-pass computes it
-  const bool in_kernel = out_dtype == PICO_BF16 && dq != nullptr && desc->Sq > 0;
-  if (!in_kernel) {
-    if (int rc = pico_attn_bwd_preprocess(desc, dout, out, out_dtype, delta, nullptr, stream)) return rc;
-    return run_bwd("pico_attn_bwd_fused", desc, q, k, v, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype,
-                   dq_accumulate, dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
-  }
-  return run_bwd("pico_attn_bwd_fused", desc, q, k, v, dout, lse, delta, out, delta, dq, dq_stride, dq_dtype, dq_accumulate,
-                 dk, dv, dkv_stride, dkv_dtype, dkv_accumulate, stream);
+  const char* fn = "pico_attn_bwd_fused";
+  if (int rc = check_attn_desc(fn, desc)) return rc;
+  if (dkv_accumulate && dkv_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
+  const pico_kv_chunks kv = one_chunk(desc, k, v, dk, dv, dkv_accumulate);
+  return run_bwd_with_out(fn, desc, q, &kv, dout, out, out_dtype, lse, delta, dq, dq_stride, dq_dtype, dq_accumulate,
+                          dkv_stride, dkv_dtype, stream, nullptr);
 }
 
 extern "C" int pico_attn_bwd_rope(const pico_attn_desc* desc, const void* q_rot, const void* k_rot, const void* v,
                                   const void* dout, const void* out, const float* lse, float* delta, void* dq,
-                                  const int64_t* dq_stride, int dq_dtype, void* dk, void* dv, const int64_t* dkv_stride,
-                                  int dkv_dtype, const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset,
-                                  void* stream) {
+                                  const int64_t* dq_stride, int dq_dtype, int dq_accumulate, void* dk, void* dv,
+                                  const int64_t* dkv_stride, int dkv_dtype, int dkv_accumulate,
+                                  const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset, void* stream) {
   const char* fn = "pico_attn_bwd_rope";
   if (int rc = check_attn_desc(fn, desc)) return rc;
   if (desc->B == 0) return PICO_OK;
-  if (q_pos_offset < 0 || k_pos_offset < 0) return fail(PICO_ERR_SHAPE, "%s: position offsets must be >= 0", fn);
-  const int64_t last = (static_cast<int64_t>(q_pos_offset) + desc->Sq > static_cast<int64_t>(k_pos_offset) + desc->Sk
-                            ? static_cast<int64_t>(q_pos_offset) + desc->Sq
-                            : static_cast<int64_t>(k_pos_offset) + desc->Sk) - 1;
-  if (int rc = check_rope_tables(fn, rope, desc->D, last)) return rc;
+  RopeArgs r;
+  if (int rc = rope_args(fn, desc, rope, q_pos_offset, k_pos_offset, r)) return rc;
   if (!dq || !dk || !dv) return fail(PICO_ERR_NULL, "%s: dq, dk and dv are required", fn);
-  if (desc->Sq > 0 && (!out || !delta)) return fail(PICO_ERR_NULL, "%s: out and delta are required", fn);
-  const RopeArgs r{rope->cos, rope->sin, rope->pitch, rope->dtype == PICO_F32, q_pos_offset, k_pos_offset};
-  // the dQ kernel computes delta from the bf16 forward output in its prologue and runs before the dK/dV kernel
-  return run_bwd(fn, desc, q_rot, k_rot, v, dout, lse, delta, out, delta, dq, dq_stride, dq_dtype, 0, dk, dv, dkv_stride,
-                 dkv_dtype, 0, stream, &r);
+  if (dkv_accumulate && dkv_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
+  const pico_kv_chunks kv = one_chunk(desc, k_rot, v, dk, dv, dkv_accumulate);
+  return run_bwd_with_out(fn, desc, q_rot, &kv, dout, out, PICO_BF16, lse, delta, dq, dq_stride, dq_dtype, dq_accumulate,
+                          dkv_stride, dkv_dtype, stream, &r);
+}
+
+extern "C" int pico_attn_bwd_chunks(const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, const void* dout,
+                                    const void* out, int out_dtype, const float* lse, float* delta, void* dq,
+                                    const int64_t* dq_stride, int dq_dtype, int dq_accumulate, const int64_t* dkv_stride,
+                                    int dkv_dtype, const pico_rope_tables* rope, int q_pos_offset, int k_pos_offset,
+                                    void* stream) {
+  const char* fn = "pico_attn_bwd_chunks";
+  if (int rc = check_attn_desc(fn, desc)) return rc;
+  if (!kv) return fail(PICO_ERR_NULL, "%s: the chunk list is NULL", fn);
+  if (desc->B == 0) return PICO_OK;
+  RopeArgs r;
+  if (rope) {
+    if (int rc = rope_args(fn, desc, rope, q_pos_offset, k_pos_offset, r)) return rc;
+  }
+  if (out)
+    return run_bwd_with_out(fn, desc, q, kv, dout, out, out_dtype, lse, delta, dq, dq_stride, dq_dtype, dq_accumulate, dkv_stride,
+                            dkv_dtype, stream, rope ? &r : nullptr);
+  return run_bwd(fn, desc, q, kv, dout, lse, delta, nullptr, nullptr, dq, dq_stride, dq_dtype, dq_accumulate, dkv_stride,
+                 dkv_dtype, stream, rope ? &r : nullptr);
 }

@@ -258,17 +258,68 @@ __device__ __forceinline__ void rope_unrotate_acc(f32x16 (&acc)[D / 32], const R
     }
 }
 
+// K / V as a list of equally long chunks that lie one after another along the key axis: key j of the launch is row
+// j % len of chunk j / len.  One chunk of len = Sk is the plain case.  With several chunks len is a multiple of every
+// kernel's staged key tile (128), so no tile straddles two chunks.
+constexpr int kMaxChunks = PICO_MAX_KV_CHUNKS;
+struct KvChunks {
+  const __bf16* k[kMaxChunks];
+  const __bf16* v[kMaxChunks];
+  int count, len;
+};
+
 struct AttnParams {
-  const __bf16* q; const __bf16* k; const __bf16* v;
+  const __bf16* q;
+  KvChunks kv;
   int B, Hq, Hkv, Sq, Sk;
   int causal, q_offset;
   float sm_scale;
   int64_t qs[3], ks[3], vs[3], os[3];
 };
 
+// A cursor over the key tiles of KT keys, in order, across the chunks: wave-uniform, so it lives in scalar registers;
+// stepping inside a chunk is four adds, a new chunk re-reads its base addresses from the kernel arguments.
+template <int D>
+struct KvCursor {
+  const char *k, *v;            // first row of the next tile
+  uint32_t k_left, v_left;      // bytes from there to the end of the chunk's rows of this head
+  uint32_t k_step, v_step;
+  int tiles_left, chunk, tiles_per_chunk;
+  int64_t k_head, v_head;       // element offset of the (batch, kv head) inside every chunk
+  __device__ __forceinline__ void open(const AttnParams& a, int chunk_, int b, int hkv, int KT) {
+    chunk = chunk_;
+    k_head = b * a.ks[0] + hkv * a.ks[1];
+    v_head = b * a.vs[0] + hkv * a.vs[1];
+    k_step = static_cast<uint32_t>(KT * a.ks[2] * 2);
+    v_step = static_cast<uint32_t>(KT * a.vs[2] * 2);
+    tiles_per_chunk = (a.kv.len + KT - 1) / KT;
+    enter(a);
+  }
+  __device__ __forceinline__ void enter(const AttnParams& a) {
+    k = reinterpret_cast<const char*>(a.kv.k[chunk] + k_head);
+    v = reinterpret_cast<const char*>(a.kv.v[chunk] + v_head);
+    k_left = span_bytes(a.kv.len, a.ks[2], D);
+    v_left = span_bytes(a.kv.len, a.vs[2], D);
+    tiles_left = tiles_per_chunk;
+  }
+  __device__ __forceinline__ void next(const AttnParams& a) {
+    if (--tiles_left == 0 && chunk + 1 < a.kv.count) {
+      ++chunk;
+      enter(a);
+    } else {
+      k += k_step;  k_left -= k_step;
+      v += v_step;  v_left -= v_step;
+    }
+  }
+};
+
 int check_attn_desc(const char* fn, const pico_attn_desc* d);
 // tables usable for head_dim D and positions 0 .. last_pos?
 int check_rope_tables(const char* fn, const pico_rope_tables* t, int D, int64_t last_pos);
+// one chunk of d->Sk keys
 AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, const void* v);
+// the chunk list checked against the descriptor (count, length, tile multiple, alignment; with need_kv also that no
+// k / v pointer is NULL) and copied into `a`
+int set_chunks(const char* fn, const pico_attn_desc* d, const pico_kv_chunks* kv, AttnParams& a, bool need_kv);
 
 }  // namespace pico

@@ -23,9 +23,6 @@ struct FwdParams {
   int64_t qrs[3];  // element strides (b, h, s) of q_rot
 };
 
-#ifndef PICO_FWD_KDEPTH
-#define PICO_FWD_KDEPTH (D >= 128 ? 2 : 0)
-#endif
 // KS > 1 splits the keys of a staged tile over KS waves that share the same queries (NW / KS waves cover the queries):
 // for launches with about one wave per SIMD, where a wave's S -> softmax -> PV chain per key tile is not hidden by
 // anything, this multiplies the waves in flight and divides each chain's length by KS.  The KS partial (m, l, O)
@@ -39,7 +36,7 @@ struct FwdCfg {
   static_assert(KS == 1 || QB == 1, "key split is built for one query block per wave");
   static constexpr int BN = 64;            // keys per compute step
   static constexpr int kKT = KT;           // keys per staged LDS tile (a multiple of BN), double-buffered
-  static constexpr int kKDepth = PICO_FWD_KDEPTH;  // K fragments in flight from LDS ahead of the MFMA that uses them (0: compiler's order)
+  static constexpr int kKDepth = D >= 128 ? 2 : 0;  // K fragments in flight from LDS ahead of the MFMA that uses them (0: compiler's order)
   static constexpr int LDK = D + 8;        // K tile pitch: 16-byte row reads hit distinct banks
   // V tile pitch for the 4-row transposing reads.  At head_dim 128: 16 (mod 32) words, so that the 16-word pieces of 4
   // consecutive rows tile the 64 LDS banks (2 requests per bank, the minimum for an 8-byte read; a pitch of D + 8 gives
@@ -58,30 +55,8 @@ struct FwdCfg {
   static_assert(KT % BN == 0 && (KT * kVecPerRow) % kThreads == 0, "tile must split evenly over the threads");
 };
 
-#ifndef PICO_FWD_KT8
-#define PICO_FWD_KT8 64
-#endif
-#ifndef PICO_FWD_KT128
-#define PICO_FWD_KT128 128
-#endif
-#ifndef PICO_FWD_CFG128
-#define PICO_FWD_CFG128 128, 1, 8, PICO_FWD_KT128
-#endif
-#ifndef PICO_FWD_CFG64
-#define PICO_FWD_CFG64 64, 1, 8, PICO_FWD_KT8
-#endif
-#ifndef PICO_FWD_KS
-#define PICO_FWD_KS 2
-#endif
-// workgroups of 256 queries (8 waves) a launch must have before that size is used
-#ifndef PICO_FWD_NW8_MIN
-#define PICO_FWD_NW8_MIN 512
-#endif
-#ifndef PICO_FWD_ATTR
-#define PICO_FWD_ATTR
-#endif
 template <int D, int QB, int NW, int KT, int KS = 1>
-__global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const FwdParams p) {
+__global__ __launch_bounds__(64 * NW) void attn_fwd_kernel(const FwdParams p) {
   using C = FwdCfg<D, QB, NW, KT, KS>;
   constexpr int BM = C::BM, BN = C::BN, LDK = C::LDK, LDV = C::LDV;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -104,8 +79,6 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
   const int qw = wave % C::kQWaves, ks = wave / C::kQWaves;   // which queries, which 64-key step of a staged tile
 
   const __bf16* qbase = a.q + b * a.qs[0] + hq * a.qs[1];
-  const __bf16* kbase = a.k + b * a.ks[0] + hkv * a.ks[1];
-  const __bf16* vbase = a.v + b * a.vs[0] + hkv * a.vs[1];
 
   // ---- Q fragments (B operand of S^T): lane = query, 8 consecutive d per 16-wide k step; fetched row-major and
   //      turned into fragments through the wave's piece of LDS (the tile buffers are filled only after the
@@ -187,20 +160,17 @@ __global__ __launch_bounds__(64 * NW) PICO_FWD_ATTR void attn_fwd_kernel(const F
     k_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.ks[2] + cv * 8) * 2);
     v_off[i] = static_cast<uint32_t>((static_cast<int64_t>(r) * a.vs[2] + cv * 8) * 2);
   }
-  // a cursor walks the key tiles in order: stepping it is four scalar adds instead of 64-bit multiplies
-  const char* k_ptr = reinterpret_cast<const char*>(kbase);
-  const char* v_ptr = reinterpret_cast<const char*>(vbase);
-  uint32_t k_left = span_bytes(a.Sk, a.ks[2], D), v_left = span_bytes(a.Sk, a.vs[2], D);
-  const uint32_t k_step = static_cast<uint32_t>(KT * a.ks[2] * 2), v_step = static_cast<uint32_t>(KT * a.vs[2] * 2);
+  // a cursor walks the key tiles in order (and from chunk to chunk): stepping it is a few scalar adds
+  KvCursor<D> cur;
+  cur.open(a, 0, b, hkv, KT);
   auto load_tile = [&]() {  // the next tile of KT keys
-    const buffer_rsrc kb = make_buffer(k_ptr, k_left), vb = make_buffer(v_ptr, v_left);
+    const buffer_rsrc kb = make_buffer(cur.k, cur.k_left), vb = make_buffer(cur.v, cur.v_left);
 #pragma unroll
     for (int i = 0; i < C::kLoads; ++i) {
       kreg[i] = buffer_load_b128(kb, k_off[i]);
       vreg[i] = buffer_load_b128(vb, v_off[i]);
     }
-    k_ptr += k_step;  k_left -= k_step;
-    v_ptr += v_step;  v_left -= v_step;
+    cur.next(a);
   };
   auto store_tile = [&](int buf) {
     __bf16* sK = smem + buf * C::kTileElems;
@@ -451,9 +421,8 @@ int check_attn_desc(const char* fn, const pico_attn_desc* d) {
     for (int i = 0; i < 3; ++i)
       if (st[i] < 0 || st[i] % 8 != 0)
         return fail(PICO_ERR_STRIDE, "%s: strides must be non-negative multiples of 8 elements", fn);
-  // the kernels address one head's rows through 32-bit byte offsets
-  const int64_t spans[4] = {(d->Sq - 1) * d->q_stride[2], (d->Sk - 1) * d->k_stride[2], (d->Sk - 1) * d->v_stride[2],
-                            (d->Sq - 1) * d->o_stride[2]};
+  // the kernels address one head's rows through 32-bit byte offsets (the key side is checked per chunk, set_chunks)
+  const int64_t spans[2] = {(d->Sq - 1) * d->q_stride[2], (d->Sq - 1) * d->o_stride[2]};
   for (int64_t span : spans)
     if ((span + d->D) * 2 >= (1LL << 32))
       return fail(PICO_ERR_STRIDE, "%s: the rows of one head must span less than 4 GiB", fn);
@@ -474,8 +443,11 @@ int check_rope_tables(const char* fn, const pico_rope_tables* t, int D, int64_t 
 AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, const void* v) {
   AttnParams a;
   a.q = static_cast<const __bf16*>(q);
-  a.k = static_cast<const __bf16*>(k);
-  a.v = static_cast<const __bf16*>(v);
+  for (int c = 0; c < kMaxChunks; ++c) a.kv.k[c] = a.kv.v[c] = nullptr;
+  a.kv.k[0] = static_cast<const __bf16*>(k);
+  a.kv.v[0] = static_cast<const __bf16*>(v);
+  a.kv.count = 1;
+  a.kv.len = d->Sk;
   a.B = d->B; a.Hq = d->Hq; a.Hkv = d->Hkv; a.Sq = d->Sq; a.Sk = d->Sk;
   a.causal = d->causal != 0;
   a.q_offset = d->q_offset;
@@ -486,26 +458,62 @@ AttnParams make_params(const pico_attn_desc* d, const void* q, const void* k, co
   return a;
 }
 
+int set_chunks(const char* fn, const pico_attn_desc* d, const pico_kv_chunks* kv, AttnParams& a, bool need_kv) {
+  if (!kv) return fail(PICO_ERR_NULL, "%s: the chunk list is NULL", fn);
+  if (kv->count < 1 || kv->count > kMaxChunks)
+    return fail(PICO_ERR_SHAPE, "%s: %d chunks (1 to %d supported)", fn, kv->count, kMaxChunks);
+  if (kv->chunk_len < 0 || static_cast<int64_t>(kv->count) * kv->chunk_len != d->Sk)
+    return fail(PICO_ERR_SHAPE, "%s: %d chunks of %d keys do not make Sk=%d", fn, kv->count, kv->chunk_len, d->Sk);
+  if (kv->count > 1 && kv->chunk_len % 128 != 0)
+    return fail(PICO_ERR_SHAPE, "%s: with several chunks the chunk length (%d) must be a multiple of 128", fn, kv->chunk_len);
+  // a chunk is addressed through the same 32-bit window as a whole tensor
+  if (((kv->chunk_len - 1) * std::max(d->k_stride[2], d->v_stride[2]) + d->D) * 2 >= (1LL << 32))
+    return fail(PICO_ERR_STRIDE, "%s: the rows of one head must span less than 4 GiB", fn);
+  for (int c = 0; c < kv->count; ++c) {
+    if (need_kv && (!kv->k[c] || !kv->v[c])) return fail(PICO_ERR_NULL, "%s: k / v of chunk %d are NULL", fn, c);
+    if (!aligned16(kv->k[c]) || !aligned16(kv->v[c]) || !aligned16(kv->dk[c]) || !aligned16(kv->dv[c]))
+      return fail(PICO_ERR_ALIGN, "%s: chunk %d: k, v, dk and dv must be 16-byte aligned", fn, c);
+    a.kv.k[c] = static_cast<const __bf16*>(kv->k[c]);
+    a.kv.v[c] = static_cast<const __bf16*>(kv->v[c]);
+  }
+  a.kv.count = kv->count;
+  a.kv.len = kv->chunk_len;
+  return PICO_OK;
+}
+
 }  // namespace pico
 
 using namespace pico;
 
 namespace {
 
-int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const void* k, const void* v, void* out, float* lse,
+// rows of [B, H, S, D] memory addressed by `st` must not overlap: every stride spans what lies inside it
+bool rows_disjoint(const int64_t* st, int B, int H, int S, int D) {
+  struct Dim { int64_t stride; int extent; } dims[3] = {{st[0], B}, {st[1], H}, {st[2], S}};
+  std::sort(dims, dims + 3, [](const Dim& x, const Dim& y) { return x.stride < y.stride; });
+  int64_t span = D;   // elements covered by the dimensions handled so far
+  for (const Dim& d : dims) {
+    if (d.extent <= 1) continue;
+    if (d.stride < span) return false;
+    span = d.stride * (d.extent - 1) + span;
+  }
+  return true;
+}
+
+int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, void* out, float* lse,
             int out_dtype, int merge, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
             const int64_t* q_rot_stride, void* stream) {
   if (int rc = check_attn_desc(fn, desc)) return rc;
   if (out_dtype != PICO_BF16 && out_dtype != PICO_F32)
     return fail(PICO_ERR_DTYPE, "%s: out dtype code %d not supported", fn, out_dtype);
   if (merge && out_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: merge needs an fp32 running out", fn);
-  if (desc->B == 0 || desc->Sq == 0) return PICO_OK;
-  if (!q || !out || !lse || (desc->Sk > 0 && (!k || !v)))
-    return fail(PICO_ERR_NULL, "%s: q, k, v, out and lse are required", fn);
-  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out) || !aligned16(q_rot))
-    return fail(PICO_ERR_ALIGN, "%s: q, k, v, out and q_rot must be 16-byte aligned", fn);
   FwdParams p;
-  p.a = make_params(desc, q, k, v);
+  p.a = make_params(desc, q, nullptr, nullptr);
+  if (int rc = set_chunks(fn, desc, kv, p.a, desc->B > 0 && desc->Sq > 0 && desc->Sk > 0)) return rc;
+  if (desc->B == 0 || desc->Sq == 0) return PICO_OK;
+  if (!q || !out || !lse) return fail(PICO_ERR_NULL, "%s: q, out and lse are required", fn);
+  if (!aligned16(q) || !aligned16(out) || !aligned16(q_rot))
+    return fail(PICO_ERR_ALIGN, "%s: q, out and q_rot must be 16-byte aligned", fn);
   p.out = out;
   p.lse = lse;
   p.out_f32 = out_dtype == PICO_F32;
@@ -524,6 +532,8 @@ int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
           return fail(PICO_ERR_STRIDE, "%s: q_rot strides must be non-negative multiples of 8 elements", fn);
         p.qrs[i] = q_rot_stride[i];
       }
+      if (!rows_disjoint(q_rot_stride, desc->B, desc->Hq, desc->Sq, desc->D))
+        return fail(PICO_ERR_STRIDE, "%s: q_rot strides make rows overlap (every stride must span what lies inside it)", fn);
       p.q_rot = static_cast<__bf16*>(q_rot);
     }
   }
@@ -539,36 +549,53 @@ int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const voi
     // block): the waves of a workgroup then do nearly equal work, and workgroups of eight waves, which share every
     // staged tile among twice as many waves, pay even where the launch has few of them
     const bool rectangular = !desc->causal || desc->q_offset >= desc->Sq;
-    if (groups(256) >= PICO_FWD_NW8_MIN) rc = launch<PICO_FWD_CFG64>(p, s);
+    if (groups(256) >= 512) rc = launch<64, 1, 8, 64>(p, s);
     else if (groups(128) >= 512) {
       // (measured at B8, 256 queries x 1024 keys of every head: 26.9 us with eight waves, 30.1 us with four)
-      if (rectangular && groups(256) >= 256) rc = launch<PICO_FWD_CFG64>(p, s);
+      if (rectangular && groups(256) >= 256) rc = launch<64, 1, 8, 64>(p, s);
       else rc = launch<64, 1, 4, 64>(p, s);
     }
     // few waves in all: two waves per 32 queries, 64 keys of every 128 each -- in workgroups of eight waves (128 queries)
     // when those still cover the CUs and the launch is rectangular (one rank's share of configs[1]: 19.8 -> 16.9 us for
     // rank 3 of 4; on a whole causal sequence, or with 256 keys, the smaller workgroups are a few percent faster)
     else if (groups(128) >= 256 && rectangular && visible_keys >= 512) rc = launch<64, 1, 8, 128, 2>(p, s);
-    else rc = launch<64, 1, 4, 128, PICO_FWD_KS>(p, s);
+    else rc = launch<64, 1, 4, 128, 2>(p, s);
   } else {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
-    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<PICO_FWD_CFG128>(p, s);
+    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<128, 1, 8, 128>(p, s);
     else rc = launch<128, 1, 4, 64>(p, s);
   }
   if (rc) return rc;
   return check_launch(fn);
 }
 
+pico_kv_chunks one_chunk(const pico_attn_desc* desc, const void* k, const void* v) {
+  pico_kv_chunks kv = {};
+  kv.count = 1;
+  kv.chunk_len = desc ? desc->Sk : 0;
+  kv.k[0] = k;
+  kv.v[0] = v;
+  return kv;
+}
+
 }  // namespace
 
 extern "C" int pico_attn_fwd(const pico_attn_desc* desc, const void* q, const void* k, const void* v, void* out,
                              float* lse, int out_dtype, int merge, void* stream) {
-  return run_fwd("pico_attn_fwd", desc, q, k, v, out, lse, out_dtype, merge, nullptr, 0, nullptr, nullptr, stream);
+  const pico_kv_chunks kv = one_chunk(desc, k, v);
+  return run_fwd("pico_attn_fwd", desc, q, &kv, out, lse, out_dtype, merge, nullptr, 0, nullptr, nullptr, stream);
 }
 
 extern "C" int pico_attn_fwd_rope(const pico_attn_desc* desc, const void* q, const void* k_rot, const void* v, void* out,
-                                  float* lse, int out_dtype, const pico_rope_tables* rope, int q_pos_offset, void* q_rot,
-                                  const int64_t* q_rot_stride, void* stream) {
+                                  float* lse, int out_dtype, int merge, const pico_rope_tables* rope, int q_pos_offset,
+                                  void* q_rot, const int64_t* q_rot_stride, void* stream) {
   if (!rope) return fail(PICO_ERR_NULL, "pico_attn_fwd_rope: the tables are required");
-  return run_fwd("pico_attn_fwd_rope", desc, q, k_rot, v, out, lse, out_dtype, 0, rope, q_pos_offset, q_rot, q_rot_stride, stream);
+  const pico_kv_chunks kv = one_chunk(desc, k_rot, v);
+  return run_fwd("pico_attn_fwd_rope", desc, q, &kv, out, lse, out_dtype, merge, rope, q_pos_offset, q_rot, q_rot_stride, stream);
+}
+
+extern "C" int pico_attn_fwd_chunks(const pico_attn_desc* desc, const void* q, const pico_kv_chunks* kv, void* out,
+                                    float* lse, int out_dtype, int merge, const pico_rope_tables* rope, int q_pos_offset,
+                                    void* q_rot, const int64_t* q_rot_stride, void* stream) {
+  return run_fwd("pico_attn_fwd_chunks", desc, q, kv, out, lse, out_dtype, merge, rope, q_pos_offset, q_rot, q_rot_stride, stream);
 }

@@ -35,7 +35,7 @@ import torch.nn.functional as F
 import picotron_amd.process_group_manager as pgm
 from picotron_amd.context_parallel import context_parallel
 from picotron_amd.functional import (FlashAttnFunc, FusedLinearFunc, QKVAttentionFunc, RMSNormFunc, RMSNormResidualFunc,
-                                     RotaryFunc, SwiGLUFunc, SwiGLUFusedFunc)
+                                     RotaryFunc, SwiGLUFunc, SwiGLUFusedFunc, _fused_rope)
 
 
 def apply_rotary_pos_emb(x, cos, sin):
@@ -192,12 +192,29 @@ class Attention(nn.Module):
     def forward(self, x, cos, sin, attention_mask=None, position_ids=None):
         batch_size, seq_length, _ = x.size()
         context = os.getenv("CONTEXT_PARALLEL", "0") == "1"
-        if _fused_projections() and not context and cos.size(0) >= seq_length:
+        if _fused_projections() and cos.size(0) >= seq_length:
             # one GEMM for q, k and v; RoPE, attention and their backward work on strided views of the fused buffers
             w = _fused_weight(self, "_qkv_weight", (self.q_proj, self.k_proj, self.v_proj))
             qkv = FusedLinearFunc.apply(x, w, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
-            out = QKVAttentionFunc.apply(qkv, cos, sin, self.num_local_heads, self.num_local_kv_heads, self.head_dim, True)
-            return self.out_proj(out)
+            if not context:
+                out = QKVAttentionFunc.apply(qkv, cos, sin, self.num_local_heads, self.num_local_kv_heads, self.head_dim, True)
+                return self.out_proj(out)
+            nq, nkv = self.num_local_heads * self.head_dim, self.num_local_kv_heads * self.head_dim
+            q = qkv[..., :nq].view(batch_size, seq_length, self.num_local_heads, self.head_dim).transpose(1, 2)
+            k = qkv[..., nq:nq + nkv].view(batch_size, seq_length, self.num_local_kv_heads, self.head_dim).transpose(1, 2)
+            v = qkv[..., nq + nkv:].view(batch_size, seq_length, self.num_local_kv_heads, self.head_dim).transpose(1, 2)
+            sm_scale = 1.0 / (self.head_dim ** 0.5)
+            whole_cos, whole_sin = getattr(cos, "whole_table", None), getattr(sin, "whole_table", None)
+            rank_pos = pgm.process_group_manager.cp_rank * seq_length
+            if (_fused_rope() and whole_cos is not None and whole_sin is not None
+                    and whole_cos[1] == rank_pos and whole_sin[1] == rank_pos):
+                # RoPE inside the ring: q rotated in the attention forward at the rank's absolute positions, k by one
+                # launch before its chunk is published, dq / dk un-rotated in the backward kernels' epilogues
+                out = context_parallel.ring_attention(q, k, v, sm_scale, True, rope=(whole_cos[0], whole_sin[0]))
+            else:
+                out = context_parallel.ring_attention(apply_rotary_pos_emb(q, cos, sin), apply_rotary_pos_emb(k, cos, sin), v,
+                                                      sm_scale, True)
+            return self.out_proj(out.transpose(1, 2).reshape(batch_size, seq_length, nq))
         # [B,S,H*D] -> [B,H,S,D] views over [B,S,H,D] memory; the kernels take the strides as they are
         q = self.q_proj(x).view(batch_size, seq_length, self.num_local_heads, self.head_dim).transpose(1, 2)
         k = self.k_proj(x).view(batch_size, seq_length, self.num_local_kv_heads, self.head_dim).transpose(1, 2)

@@ -10,7 +10,7 @@ from typing import Optional, Tuple
 import torch
 
 from . import _lib
-from ._lib import PICO_BF16, PICO_F32, AttnDesc, RopeTables, check
+from ._lib import MAX_KV_CHUNKS, PICO_BF16, PICO_F32, AttnDesc, KvChunks, RopeTables, check
 
 _DT = {torch.bfloat16: PICO_BF16, torch.float32: PICO_F32}
 
@@ -249,32 +249,41 @@ def _rope_tables(cos: torch.Tensor, sin: torch.Tensor) -> RopeTables:
 
 
 def attn_fwd_rope(q, k_rot, v, cos, sin, sm_scale: float, causal: bool, q_offset: int = 0, q_pos_offset: int = 0,
-                  want_q_rot: bool = True, out_dtype=torch.bfloat16, bshd_out: bool = True):
+                  want_q_rot: bool = True, out_dtype=torch.bfloat16, bshd_out: bool = True, out=None, lse=None,
+                  merge: bool = False, q_rot=None):
     """RoPE on q inside the attention forward (k_rot must be rotated already): returns (out, lse, q_rot or None); q_rot is
-    the rotated q, laid out like q, for attn_bwd_rope.  One chunk, no merge."""
-    _dev(q, k_rot, v)
+    the rotated q, laid out like q, for attn_bwd_rope.  merge=True continues from the running fp32 (out, lse) given, as
+    attn_fwd does: one step of a ring whose queries sit at positions q_pos_offset .."""
+    _dev(q, k_rot, v, out, lse, q_rot)
     q, k_rot, v = _attn_in(q, "q"), _attn_in(k_rot, "k"), _attn_in(v, "v")
     B, Hq, Sq, D = q.shape
     if k_rot.shape != v.shape or k_rot.size(0) != B or k_rot.size(3) != D:
         raise RuntimeError(f"attention: shape mismatch q{tuple(q.shape)} k{tuple(k_rot.shape)} v{tuple(v.shape)}")
-    out = empty_bshd(B, Hq, Sq, D, out_dtype, q.device) if bshd_out else torch.empty(B, Hq, Sq, D, dtype=out_dtype, device=q.device)
-    lse = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
-    q_rot = None
+    if merge and (out is None or lse is None or out.dtype != torch.float32):
+        raise RuntimeError("attn_fwd_rope(merge=True) needs the running fp32 out and lse")
+    if out is None:
+        out = empty_bshd(B, Hq, Sq, D, out_dtype, q.device) if bshd_out else torch.empty(B, Hq, Sq, D, dtype=out_dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+    if not lse.is_contiguous() or lse.dtype != torch.float32 or out.stride(-1) != 1:
+        raise RuntimeError("attn_fwd_rope: lse must be contiguous fp32 and out must have a unit D stride")
     qrs = None
-    if want_q_rot:
+    if want_q_rot and q_rot is None:
         q_rot = empty_bshd(B, Hq, Sq, D, q.dtype, q.device)
+    if q_rot is not None:
         qrs = (ctypes.c_int64 * 3)(*q_rot.stride()[:3])
     tables = _rope_tables(cos, sin)
     d = _desc(q, k_rot, v, out, sm_scale, causal, q_offset)
     check(_lib.lib().pico_attn_fwd_rope(ctypes.byref(d), _ptr(q), _ptr(k_rot), _ptr(v), _ptr(out), _ptr(lse), _dt(out, "attn out"),
-                                        ctypes.byref(tables), int(q_pos_offset), _ptr(q_rot), qrs, _stream()))
+                                        int(merge), ctypes.byref(tables), int(q_pos_offset), _ptr(q_rot), qrs, _stream()))
     return out, lse, q_rot
 
 
 def attn_bwd_rope(dout, q_rot, k_rot, v, out, lse, cos, sin, sm_scale: float, causal: bool, dq, dk, dv, q_offset: int = 0,
-                  q_pos_offset: int = 0, k_pos_offset: int = 0):
-    """Backward of "rotate q and k, attend" for one chunk: writes dq / dk (gradients of the UN-rotated q and k: RoPE's
-    backward runs in the kernels' epilogues) and dv into the given buffers (any strides with a unit D stride)."""
+                  q_pos_offset: int = 0, k_pos_offset: int = 0, dq_accumulate: bool = False, dkv_accumulate: bool = False):
+    """Backward of "rotate q and k, attend": writes (or, with the accumulate flags, adds to the fp32) dq / dk -- gradients
+    of the UN-rotated q and k: RoPE's backward runs in the kernels' epilogues -- and dv in the given buffers (any strides
+    with a unit D stride)."""
     _dev(dout, q_rot, k_rot, v, out, lse, dq, dk, dv)
     q_rot, k_rot, v, dout = _attn_in(q_rot, "q"), _attn_in(k_rot, "k"), _attn_in(v, "v"), _attn_in(dout, "dout")
     if out.stride() != dout.stride():
@@ -290,9 +299,128 @@ def attn_bwd_rope(dout, q_rot, k_rot, v, out, lse, cos, sin, sm_scale: float, ca
     dqs = (ctypes.c_int64 * 3)(*dq.stride()[:3])
     dks = (ctypes.c_int64 * 3)(*dk.stride()[:3])
     check(_lib.lib().pico_attn_bwd_rope(ctypes.byref(d), _ptr(q_rot), _ptr(k_rot), _ptr(v), _ptr(dout), _ptr(out),
-                                        _ptr(lse.contiguous()), _ptr(delta), _ptr(dq), dqs, _dt(dq, "dq"), _ptr(dk), _ptr(dv), dks,
-                                        _dt(dk, "dk/dv"), ctypes.byref(tables), int(q_pos_offset), int(k_pos_offset), _stream()))
+                                        _ptr(lse.contiguous()), _ptr(delta), _ptr(dq), dqs, _dt(dq, "dq"), int(dq_accumulate),
+                                        _ptr(dk), _ptr(dv), dks, _dt(dk, "dk/dv"), int(dkv_accumulate), ctypes.byref(tables),
+                                        int(q_pos_offset), int(k_pos_offset), _stream()))
     return dq, dk, dv
+
+
+# ---- all ring steps of one rank in one launch: K / V as a list of equally shaped chunk tensors
+def chunks_fit_one_launch(ks, vs) -> bool:
+    """True if the chunk tensors can go to the chunk-list entry points as they are: at most 16 bf16 chunks of one shape
+    and one stride triple (k's may differ from v's), unit D stride, strides that are multiples of 8, and -- with several
+    chunks -- a chunk length that is a multiple of 128 (no staged key tile straddles two chunks)."""
+    if not ks or len(ks) != len(vs) or len(ks) > MAX_KV_CHUNKS:
+        return False
+    k0, v0 = ks[0], vs[0]
+    if k0.dim() != 4 or (len(ks) > 1 and k0.size(2) % 128 != 0):
+        return False
+    for k, v in zip(ks, vs):
+        if (k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16 or k.shape != k0.shape or v.shape != k0.shape
+                or k.stride() != k0.stride() or v.stride() != v0.stride() or k.stride(-1) != 1 or v.stride(-1) != 1
+                or any(s % 8 for s in k.stride()[:3]) or any(s % 8 for s in v.stride()[:3])
+                or k.data_ptr() % 16 or v.data_ptr() % 16 or not k.is_cuda or not v.is_cuda):
+            return False
+    return True
+
+
+def _kv_chunks(ks, vs, dks=None, dvs=None, accumulate=None) -> KvChunks:
+    c = KvChunks()
+    c.count, c.chunk_len = len(ks), ks[0].size(2)
+    mask = 0
+    for i, (k, v) in enumerate(zip(ks, vs)):
+        c.k[i], c.v[i] = k.data_ptr(), v.data_ptr()
+        if dks is not None and dks[i] is not None:
+            c.dk[i], c.dv[i] = dks[i].data_ptr(), dvs[i].data_ptr()
+            if accumulate is not None and accumulate[i]:
+                mask |= 1 << i
+    c.accumulate_mask = mask
+    return c
+
+
+def _chunk_desc(q, ks, vs, o, sm_scale, causal, q_offset) -> AttnDesc:
+    d = _desc(q, ks[0], vs[0], o, sm_scale, causal, q_offset)
+    d.Sk = len(ks) * ks[0].size(2)
+    return d
+
+
+def attn_fwd_chunks(q, ks, vs, sm_scale: float, causal: bool, q_offset: int = 0, out=None, lse=None, merge: bool = False,
+                    out_dtype=torch.bfloat16, bshd_out: bool = False, rope=None, q_pos_offset: int = 0,
+                    want_q_rot: bool = False):
+    """attn_fwd over K / V given as lists of chunk tensors (see chunks_fit_one_launch) that follow each other along the
+    key axis: key j sits at position j of the concatenation, which is never materialised.  rope = (cos, sin): q is
+    rotated inside the kernel (the chunks' k must be rotated already).  Returns (out, lse, q_rot or None)."""
+    _dev(q, out, lse)
+    if not chunks_fit_one_launch(ks, vs):
+        raise RuntimeError("attn_fwd_chunks: the chunks do not fit one launch (see chunks_fit_one_launch)")
+    q = _attn_in(q, "q")
+    B, Hq, Sq, D = q.shape
+    if ks[0].size(0) != B or ks[0].size(3) != D:
+        raise RuntimeError(f"attention: shape mismatch q{tuple(q.shape)} k{tuple(ks[0].shape)}")
+    if merge and (out is None or lse is None or out.dtype != torch.float32):
+        raise RuntimeError("attn_fwd_chunks(merge=True) needs the running fp32 out and lse")
+    if out is None:
+        out = empty_bshd(B, Hq, Sq, D, out_dtype, q.device) if bshd_out else torch.empty(B, Hq, Sq, D, dtype=out_dtype, device=q.device)
+    if lse is None:
+        lse = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+    if not lse.is_contiguous() or lse.dtype != torch.float32 or out.stride(-1) != 1:
+        raise RuntimeError("attn_fwd_chunks: lse must be contiguous fp32 and out must have a unit D stride")
+    d = _chunk_desc(q, ks, vs, out, sm_scale, causal, q_offset)
+    kv = _kv_chunks(ks, vs)
+    tables = q_rot = qrs = None
+    if rope is not None:
+        tables = ctypes.byref(_rope_tables(*rope))
+        if want_q_rot:
+            q_rot = empty_bshd(B, Hq, Sq, D, q.dtype, q.device)
+            qrs = (ctypes.c_int64 * 3)(*q_rot.stride()[:3])
+    check(_lib.lib().pico_attn_fwd_chunks(ctypes.byref(d), _ptr(q), ctypes.byref(kv), _ptr(out), _ptr(lse), _dt(out, "attn out"),
+                                          int(merge), tables, int(q_pos_offset), _ptr(q_rot), qrs, _stream()))
+    return out, lse, q_rot
+
+
+def attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale: float, causal: bool, q_offset: int = 0, dq=None, dks=None, dvs=None,
+                    dq_accumulate: bool = False, dkv_accumulate=None, out=None, delta=None, rope=None,
+                    q_pos_offset: int = 0, k_pos_offset: int = 0):
+    """attn_bwd over a chunk list.  dks / dvs: per chunk a gradient buffer (all of one dtype and stride triple) or None
+    (not wanted); dkv_accumulate: per chunk, add to the fp32 buffer instead of writing it.  dq None: not wanted.  With
+    `out` (forward output) delta is computed inside the call, otherwise `delta` must be given.  rope = (cos, sin): q and
+    the chunks' k are rotated tensors, dq / dk leave un-rotated.  Returns delta."""
+    _dev(dout, q, lse, dq, out, delta)
+    if not chunks_fit_one_launch(ks, vs):
+        raise RuntimeError("attn_bwd_chunks: the chunks do not fit one launch (see chunks_fit_one_launch)")
+    q, dout = _attn_in(q, "q"), _attn_in(dout, "dout")
+    B, Hq, Sq, D = q.shape
+    if out is not None and out.stride() != dout.stride():
+        out = _like_strided(out, dout)
+    if delta is None:
+        if out is None:
+            raise RuntimeError("attn_bwd_chunks: delta (or out, to compute it) is required")
+        delta = torch.empty(B, Hq, Sq, dtype=torch.float32, device=q.device)
+    if not (delta.is_contiguous() and delta.dtype == torch.float32 and delta.numel() == B * Hq * Sq):
+        raise RuntimeError("attn_bwd_chunks: delta must be contiguous fp32 [B,H,S]")
+    given = [t for t in (dks or []) if t is not None]
+    dkv_dt, dks_arr = PICO_F32, None
+    if given:
+        g0 = given[0]
+        for a, b_ in zip(dks, dvs):
+            if (a is None) != (b_ is None):
+                raise RuntimeError("attn_bwd_chunks: dk and dv of a chunk must be given together")
+            if a is not None and (a.dtype != g0.dtype or b_.dtype != g0.dtype or a.stride() != g0.stride() or b_.stride() != g0.stride()
+                                  or a.stride(-1) != 1 or a.shape != ks[0].shape or not a.is_cuda or not b_.is_cuda):
+                raise RuntimeError("attn_bwd_chunks: all dk / dv buffers must share dtype and strides (unit D stride) and have the chunks' shape")
+        dkv_dt = _dt(g0, "dk/dv")
+        dks_arr = (ctypes.c_int64 * 3)(*g0.stride()[:3])
+    if dq is not None and dq.stride(-1) != 1:
+        raise RuntimeError("attn_bwd_chunks: dq needs a unit D stride")
+    dqs = (ctypes.c_int64 * 3)(*(dq.stride()[:3] if dq is not None else (0, 0, 0)))
+    d = _chunk_desc(q, ks, vs, dout, sm_scale, causal, q_offset)
+    kv = _kv_chunks(ks, vs, dks if given else None, dvs, dkv_accumulate)
+    tables = ctypes.byref(_rope_tables(*rope)) if rope is not None else None
+    check(_lib.lib().pico_attn_bwd_chunks(ctypes.byref(d), _ptr(q), ctypes.byref(kv), _ptr(dout), _ptr(out),
+                                          _dt(out, "out") if out is not None else PICO_BF16, _ptr(lse.contiguous()), _ptr(delta),
+                                          _ptr(dq), dqs, _dt(dq, "dq") if dq is not None else PICO_F32, int(dq_accumulate),
+                                          dks_arr, dkv_dt, tables, int(q_pos_offset), int(k_pos_offset), _stream()))
+    return delta
 
 
 def attn_bwd_preprocess(dout: torch.Tensor, out: torch.Tensor, dq_acc: Optional[torch.Tensor] = None,

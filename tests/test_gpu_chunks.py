@@ -1,0 +1,256 @@
+"""GPU parity of the chunk-list attention entry points (all ring steps of one rank in one launch), of RoPE inside
+the ring (merge / accumulate forms with position offsets), and of the backward at large score magnitudes.
+
+Tolerances: forward max-abs <= 2e-2 (bf16), lse <= 1e-3, gradients relative L2 <= 1e-2 against the fp32 oracle;
+where two GPU paths execute the same arithmetic in the same order they are compared bit for bit.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import layers as OL
+from oracle import ring as OR
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_l2(a, b):
+    a, b = a.double().cpu(), b.double().cpu()
+    return ((a - b).norm() / b.norm().clamp_min(1e-30)).item()
+
+
+def maxabs(a, b):
+    return (a.double().cpu() - b.double().cpu()).abs().max().item()
+
+
+@pytest.fixture(scope="module")
+def ops(device):
+    from picotron_amd import ops as _ops
+    return _ops
+
+
+def ring_inputs(B, Hq, Hkv, W, Sc, D, seed, q_scale=1.0, k_scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = (torch.randn(B, Hq, W * Sc, D, generator=g) * q_scale).to(torch.bfloat16)
+    k = (torch.randn(B, Hkv, W * Sc, D, generator=g) * k_scale).to(torch.bfloat16)
+    v = torch.randn(B, Hkv, W * Sc, D, generator=g).to(torch.bfloat16)
+    do = torch.randn(B, Hq, W * Sc, D, generator=g).to(torch.bfloat16)
+    return q, k, v, do
+
+
+def separate_chunks(t, W, device):
+    """The W chunks of t along S as tensors of their own (own allocations, as chunks published by different ranks are)."""
+    return [c.contiguous().to(device).clone() for c in t.chunk(W, dim=2)]
+
+
+# ------------------------------------------------------------------------------------ chunk lists
+CHUNK_CASES = [
+    # B, Hq, Hkv, W, Sc, D, rank, causal
+    (2, 4, 4, 4, 128, 64, 3, True),       # the last rank of four: chunks 0..3, diagonal in the last
+    (1, 4, 2, 4, 128, 64, 1, True),       # GQA, a middle rank: chunks 0..1
+    (1, 2, 2, 3, 256, 64, 2, False),      # no mask: every chunk dense
+    (1, 4, 2, 3, 128, 128, 2, True),      # head_dim 128
+    (4, 32, 32, 4, 256, 64, 3, True),     # rank 3 of 4 at the benchmark's shape (key-split workgroups of eight waves)
+    (1, 8, 2, 2, 384, 128, 1, True),      # head_dim 128, GQA, chunk length not a power of two
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,W,Sc,D,r,causal", CHUNK_CASES)
+def test_chunk_list_equals_contiguous_keys_and_oracle(ops, device, B, Hq, Hkv, W, Sc, D, r, causal):
+    """One launch over the chunk tensors of ranks 0..r (or all W without a mask) against (a) the same launch over one
+    contiguous K / V tensor -- the same tiles in the same order, so bit for bit -- and (b) the oracle's rank_forward /
+    rank_backward, which walks the ring step by step."""
+    q, k, v, do = ring_inputs(B, Hq, Hkv, W, Sc, D, seed=300 + Sc + D + r)
+    scale = 1 / math.sqrt(D)
+    n = r + 1 if causal else W
+    q_off = r * Sc if causal else 0
+    sl = slice(r * Sc, (r + 1) * Sc)
+    qd, dod = q[:, :, sl].contiguous().to(device), do[:, :, sl].contiguous().to(device)
+    ks, vs = separate_chunks(k, W, device)[:n], separate_chunks(v, W, device)[:n]
+    kc, vc = k[:, :, :n * Sc].contiguous().to(device), v[:, :, :n * Sc].contiguous().to(device)
+    assert ops.chunks_fit_one_launch(ks, vs)
+
+    out, lse, _ = ops.attn_fwd_chunks(qd, ks, vs, scale, causal, q_off)
+    out1, lse1 = ops.attn_fwd(qd, kc, vc, scale, causal, q_off)
+    assert torch.equal(out, out1) and torch.equal(lse, lse1)
+
+    rep = Hq // Hkv
+    kf = [t.float().repeat_interleave(rep, 1) for t in k.chunk(W, 2)]
+    vf = [t.float().repeat_interleave(rep, 1) for t in v.chunk(W, 2)]
+    w_o, w_l = OR.rank_forward(q[:, :, sl].float(), kf, vf, r, scale, causal)
+    assert maxabs(out, w_o) <= 2e-2 and maxabs(lse, w_l) <= 1e-3
+
+    # backward: dq in bf16, dk / dv per chunk in fp32; chunk 0 adds to what is there, the others write
+    dq = torch.empty_like(qd)
+    dks = [torch.full(t.shape, 1.5 if i == 0 else float("nan"), dtype=torch.float32, device=device) for i, t in enumerate(ks)]
+    dvs = [torch.full(t.shape, -2.0 if i == 0 else float("nan"), dtype=torch.float32, device=device) for i, t in enumerate(ks)]
+    delta = ops.attn_bwd_chunks(dod, qd, ks, vs, lse, scale, causal, q_off, dq, dks, dvs,
+                                dkv_accumulate=[i == 0 for i in range(n)], out=out)
+    dq1 = torch.empty_like(qd)
+    dk1 = torch.empty(kc.shape, dtype=torch.float32, device=device)
+    dv1 = torch.empty_like(dk1)
+    ops.attn_bwd(dod, qd, kc, vc, lse1, None, scale, causal, q_off, dq1, dk1, dv1, out=out1)
+    assert torch.equal(dq, dq1)
+    for c in range(n):
+        ref_k, ref_v = dk1[:, :, c * Sc:(c + 1) * Sc], dv1[:, :, c * Sc:(c + 1) * Sc]
+        if c == 0:   # added to what was there, in fp32
+            ref_k, ref_v = ref_k + 1.5, ref_v - 2.0
+        assert torch.equal(dks[c], ref_k) and torch.equal(dvs[c], ref_v), c
+    w_dq, contrib = OR.rank_backward(do[:, :, sl].float(), q[:, :, sl].float(), kf, vf, out.float().cpu(), lse.cpu(), r, scale, causal)
+    fold = lambda t: t.view(B, Hkv, rep, Sc, D).sum(2)
+    assert maxabs(delta, (do[:, :, sl].float() * out.float().cpu()).sum(-1)) <= 5e-2
+    assert rel_l2(dq, w_dq) <= 1e-2
+    for c in range(n):
+        base_k, base_v = (1.5, -2.0) if c == 0 else (0.0, 0.0)
+        assert rel_l2(dks[c] - base_k, fold(contrib[c][0])) <= 1e-2, c
+        assert rel_l2(dvs[c] - base_v, fold(contrib[c][1])) <= 1e-2, c
+
+
+def test_chunk_list_skips_chunks_whose_gradient_is_not_wanted(ops, device):
+    q, k, v, do = ring_inputs(1, 2, 2, 3, 128, 64, seed=11)
+    scale = 0.125
+    qd, dod = q[:, :, 256:].contiguous().to(device), do[:, :, 256:].contiguous().to(device)
+    ks, vs = separate_chunks(k, 3, device), separate_chunks(v, 3, device)
+    out, lse, _ = ops.attn_fwd_chunks(qd, ks, vs, scale, True, 256)
+    full_k = [torch.empty(t.shape, dtype=torch.float32, device=device) for t in ks]
+    full_v = [torch.empty(t.shape, dtype=torch.float32, device=device) for t in ks]
+    ops.attn_bwd_chunks(dod, qd, ks, vs, lse, scale, True, 256, None, full_k, full_v, out=out)
+    part_k = [None, torch.empty_like(full_k[1]), None]
+    part_v = [None, torch.empty_like(full_k[1]), None]
+    ops.attn_bwd_chunks(dod, qd, ks, vs, lse, scale, True, 256, None, part_k, part_v, out=out)
+    assert torch.equal(part_k[1], full_k[1]) and torch.equal(part_v[1], full_v[1])
+
+
+def test_chunk_list_rejects_what_one_launch_cannot_do(ops, device):
+    q, k, v, _ = ring_inputs(1, 2, 2, 2, 64, 64, seed=5)
+    ks, vs = separate_chunks(k, 2, device), separate_chunks(v, 2, device)
+    assert not ops.chunks_fit_one_launch(ks, vs)           # 64-key chunks: a staged tile would straddle two chunks
+    with pytest.raises(RuntimeError):
+        ops.attn_fwd_chunks(q[:, :, 64:].contiguous().to(device), ks, vs, 0.125, True, 64)
+    # the C ABI says so itself
+    import ctypes
+    from picotron_amd import _lib
+    d = ops._chunk_desc(q[:, :, 64:].contiguous().to(device), ks, vs, q[:, :, 64:].contiguous().to(device), 0.125, True, 64)
+    kv = ops._kv_chunks(ks, vs)
+    rc = _lib.lib().pico_attn_fwd_chunks(ctypes.byref(d), None, ctypes.byref(kv), None, None, 0, 0, None, 0, None, None, None)
+    assert rc == -3 and b"multiple of 128" in _lib.lib().pico_last_error()
+    one = [ks[0]], [vs[0]]
+    assert ops.chunks_fit_one_launch(*one)                 # a single chunk may have any length
+    kbad = [ks[0], ks[1][:, :, :32]]
+    assert not ops.chunks_fit_one_launch(kbad, vs)
+
+
+# ------------------------------------------------------------------------------------ RoPE inside the ring
+@pytest.mark.parametrize("D,Hq,Hkv,Sc", [(64, 4, 2, 128), (128, 4, 4, 128), (64, 2, 2, 96)])
+@pytest.mark.parametrize("table_dtype", [torch.bfloat16, torch.float32])
+def test_ring_with_rope_inside_every_rank(ops, device, D, Hq, Hkv, Sc, table_dtype):
+    """A W = 4 causal ring with RoPE at absolute positions, all ranks, two ways on the GPU:
+    (a) step by step -- pico_attn_fwd_rope rotates q at q_pos_offset = r * Sc in the first step, the later steps merge;
+        pico_attn_bwd_rope adds every block to the rank's fp32 dq and to the chunk's fp32 dk / dv with
+        k_pos_offset = c * Sc;
+    (b) one launch per rank over the chunk list (chunk lengths that are multiples of 128 only).
+    Against oracle.layers.apply_rotary_pos_emb + oracle.ring.all_ranks_forward / backward in fp32 (rotated operands
+    rounded to bf16 as the reference hands them to attention, model.py:136-137; the rounding passes gradients
+    through)."""
+    W, B = 4, 2
+    S = W * Sc
+    q, k, v, do = ring_inputs(B, Hq, Hkv, W, Sc, D, seed=900 + D + Sc)
+    scale = 1 / math.sqrt(D)
+    cos, sin = OL.get_cos_sin(S, D, 10000.0, table_dtype)
+    rep = Hq // Hkv
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    q_r = OL.apply_rotary_pos_emb(qf, cos.float(), sin.float())
+    k_r = OL.apply_rotary_pos_emb(kf, cos.float(), sin.float())
+    q_r = q_r + (q_r.detach().to(torch.bfloat16).float() - q_r.detach())
+    k_r = k_r + (k_r.detach().to(torch.bfloat16).float() - k_r.detach())
+    w_o, w_l = OR.all_ranks_forward(q_r, k_r.repeat_interleave(rep, 1), vf.repeat_interleave(rep, 1), W, scale, True)
+    gq, gk, gv = torch.autograd.grad(w_o, (qf, kf, vf), do.float())
+
+    cd, sd = cos.to(device), sin.to(device)
+    qs, dos = separate_chunks(q, W, device), separate_chunks(do, W, device)
+    ks, vs = separate_chunks(k, W, device), separate_chunks(v, W, device)
+    k_rot = [ops.rope(ks[c], cd, sd, pos_offset=c * Sc) for c in range(W)]
+
+    def run(one_launch):
+        outs, lses, dqs = [], [], []
+        dk = [torch.empty(B, Hkv, Sc, D, dtype=torch.float32, device=device) for _ in range(W)]
+        dv = [torch.empty(B, Hkv, Sc, D, dtype=torch.float32, device=device) for _ in range(W)]
+        fresh = [True] * W
+        saved = []
+        for r in range(W):
+            if one_launch:
+                out, lse, q_rot = ops.attn_fwd_chunks(qs[r], k_rot[:r + 1], vs[:r + 1], scale, True, r * Sc, rope=(cd, sd),
+                                                      q_pos_offset=r * Sc, want_q_rot=True)
+            else:
+                out32 = torch.empty(B, Hq, Sc, D, dtype=torch.float32, device=device)
+                lse = torch.empty(B, Hq, Sc, dtype=torch.float32, device=device)
+                q_rot = None
+                for step, held, runs, masked in OR.schedule(W, r, True):
+                    if not runs:
+                        continue
+                    # q is rotated by every step's prologue; only the first one leaves the rotated copy behind
+                    _, _, qr = ops.attn_fwd_rope(qs[r], k_rot[held], vs[held], cd, sd, scale, masked, 0, q_pos_offset=r * Sc,
+                                                 want_q_rot=step == 0, out=out32, lse=lse, merge=step > 0)
+                    q_rot = qr if step == 0 else q_rot
+                out = ops.convert_f32(out32, torch.bfloat16)
+            assert maxabs(q_rot, q_r.detach()[:, :, r * Sc:(r + 1) * Sc]) <= 3e-2
+            outs.append(out)
+            lses.append(lse)
+            saved.append(q_rot)
+        for r in reversed(range(W)):
+            dq = torch.empty(B, Hq, Sc, D, dtype=torch.float32, device=device)
+            if one_launch:
+                ops.attn_bwd_chunks(dos[r], saved[r], k_rot[:r + 1], vs[:r + 1], lses[r], scale, True, r * Sc, dq, dk[:r + 1], dv[:r + 1],
+                                    dkv_accumulate=[not f for f in fresh[:r + 1]], out=outs[r], rope=(cd, sd), q_pos_offset=r * Sc)
+                for c in range(r + 1):
+                    fresh[c] = False
+            else:
+                first = True
+                for step, held, runs, masked in OR.schedule(W, r, True):
+                    if not runs:
+                        continue
+                    ops.attn_bwd_rope(dos[r], saved[r], k_rot[held], vs[held], outs[r], lses[r], cd, sd, scale, masked, dq, dk[held],
+                                      dv[held], 0, q_pos_offset=r * Sc, k_pos_offset=held * Sc, dq_accumulate=not first,
+                                      dkv_accumulate=not fresh[held])
+                    first, fresh[held] = False, False
+            dqs.append(dq)
+        dqs.reverse()
+        return torch.cat(outs, 2), torch.cat(lses, 2), torch.cat(dqs, 2), torch.cat(dk, 2), torch.cat(dv, 2)
+
+    modes = [False] + ([True] if Sc % 128 == 0 else [])
+    for one_launch in modes:
+        out, lse, dq, dk, dv = run(one_launch)
+        assert maxabs(out, w_o.detach()) <= 2e-2, one_launch
+        # lse: a one-ulp flip of a bf16-rounded rotated q element moves a score by up to ~2e-3, and the kernel's
+        # rotation (fp32 tables rounded once) and the oracle's can differ by such flips
+        assert maxabs(lse, w_l.detach()) <= 2e-3, one_launch
+        assert rel_l2(dq, gq) <= 1e-2 and rel_l2(dk, gk) <= 1e-2 and rel_l2(dv, gv) <= 1e-2, one_launch
+
+
+# ------------------------------------------------------------------------------------ large scores
+@pytest.mark.parametrize("D,S,B,H", [(64, 1024, 1, 4), (128, 512, 1, 4), (64, 256, 2, 2)])
+@pytest.mark.parametrize("sigma2", [6.0, 9.0])
+def test_attn_bwd_at_large_score_magnitudes(ops, device, D, S, B, H, sigma2):
+    """q and k scaled so that the scaled scores reach |s| of 20 to 40 (N(0,1) inputs give |s| <= 6): the backward
+    recomputes P = exp(s - lse) from the forward's lse, so any rounding of the exponent that grows with |s| shows up as
+    row sums of P that are not 1 and as a gradient bias.  fp32 oracle by autograd on the same bf16 inputs."""
+    amp = math.sqrt(sigma2)
+    q, k, v, do = ring_inputs(B, H, H, 1, S, D, seed=77 + D, q_scale=amp, k_scale=amp)
+    scale = 1 / math.sqrt(D)
+    s_max = (q.float() @ k.float().transpose(-1, -2)).abs().max().item() * scale
+    assert 20.0 <= s_max <= 60.0, s_max
+    qd, kd, vd, dod = (t.to(device) for t in (q, k, v, do))
+    out, lse = ops.attn_fwd(qd, kd, vd, scale, True, 0)
+    dq, dk, dv = ops.attn_bwd(dod, qd, kd, vd, lse, None, scale, True, 0, out=out)
+    qf, kf, vf = (t.float().requires_grad_() for t in (q, k, v))
+    w_o, w_l = OR.full_attention_closed_form(qf, kf, vf, scale, True)
+    gq, gk, gv = torch.autograd.grad(w_o, (qf, kf, vf), do.float())
+    assert maxabs(out, w_o.detach()) <= 2e-2 and maxabs(lse, w_l.detach()) <= 1e-3
+    # the same bar as at small scores: the exponent is formed in fp32 from the unscaled bf16 operands
+    assert rel_l2(dq, gq) <= 1e-2 and rel_l2(dk, gk) <= 1e-2 and rel_l2(dv, gv) <= 1e-2
+    # both backward kernels recompute P on their own; they agree on it iff sum_i dq_i . q_i = sum_j dk_j . k_j
+    # (either side is sm_scale * sum_ij dS_ij q_i . k_j)
+    lhs = (dq.double().cpu() * q.double()).sum().item()
+    rhs = (dk.double().cpu() * k.double()).sum().item()
+    assert abs(lhs - rhs) <= 1e-3 * (dq.double().cpu() * q.double()).abs().sum().item()

@@ -63,12 +63,21 @@ def test_init_order_matches_oracle(pgm1, device):
     assert torch.equal(a.final_proj.weight, b.final_proj.weight)
 
 
-def test_ring_attention_func_every_rank(pgm1, device):
+@pytest.mark.parametrize("Sc,per_step", [(64, "0"), (128, "0"), (128, "1")])
+def test_ring_attention_func_every_rank(pgm1, device, Sc, per_step, monkeypatch):
     """RingAttentionFunc on virtual ranks (forward ascending, one backward over the summed loss) against
-    full-sequence causal attention in fp32."""
+    full-sequence causal attention in fp32.  Chunks of 128 keys take one launch per rank and direction over the chunk
+    list, chunks of 64 (a staged key tile would straddle two of them) and PICO_RING_PER_STEP=1 one launch per ring
+    step."""
     import picotron_amd.process_group_manager as pgm
+    from picotron_amd import ops
     from picotron_amd.context_parallel import context_parallel as cp
-    W, B, H, Hkv, Sc, D = 4, 2, 4, 2, 64, 64
+    monkeypatch.setenv("PICO_RING_PER_STEP", per_step)
+    calls = {"chunks": 0, "steps": 0}
+    real_chunks, real_fwd = ops.attn_fwd_chunks, ops.attn_fwd
+    monkeypatch.setattr(ops, "attn_fwd_chunks", lambda *a, **k: (calls.__setitem__("chunks", calls["chunks"] + 1), real_chunks(*a, **k))[1])
+    monkeypatch.setattr(ops, "attn_fwd", lambda *a, **k: (calls.__setitem__("steps", calls["steps"] + 1), real_fwd(*a, **k))[1])
+    W, B, H, Hkv, D = 4, 2, 4, 2, 64
     S = W * Sc
     g = torch.Generator().manual_seed(3)
     q, k, v, do = (torch.randn(B, h, S, D, generator=g).to(torch.bfloat16) for h in (H, Hkv, Hkv, H))
@@ -90,6 +99,10 @@ def test_ring_attention_func_every_rank(pgm1, device):
     assert out.dtype == torch.bfloat16
     assert maxabs(out, w_o) <= 2e-2
     assert rel_l2(qd.grad, gq) <= 1e-2 and rel_l2(kd.grad, gk) <= 1e-2 and rel_l2(vd.grad, gv) <= 1e-2
+    # the path that was meant ran: W launches over chunk lists, or one per executed ring step (1 + 2 + 3 + 4); rank 0
+    # reads one chunk, which fits one launch whatever its length
+    want = (0, W * (W + 1) // 2) if per_step == "1" else (W, 0) if Sc % 128 == 0 else (1, W * (W + 1) // 2 - 1)
+    assert (calls["chunks"], calls["steps"]) == want
     pgm.setup_process_group_manager(1, 1, 1, 1)
 
 
@@ -273,13 +286,19 @@ def test_smollm135m_2layer_step_matches_cpu_oracle(pgm1, device, flash_env):
     os.environ.pop("FLASH_ATTEN", None)
 
 
-def test_model_cp4_virtual_ranks_equals_cp1(pgm1, device):
-    """Four virtual cp ranks over the sequence give the same loss and gradients as one rank."""
+@pytest.mark.parametrize("seq,fused_rope", [(256, "1"), (512, "1"), (512, "0")])
+def test_model_cp4_virtual_ranks_equals_cp1(pgm1, device, seq, fused_rope, monkeypatch):
+    """Four virtual cp ranks over the sequence give the same loss and gradients as one rank.  The context-parallel
+    model takes the fused q/k/v projection with RoPE inside the ring (q rotated in the attention forward at the rank's
+    absolute positions, dq / dk un-rotated in the backward kernels; PICO_FUSED_ROPE=0: RoPE launches of their own);
+    512 tokens give chunks of 128 (one launch per rank over the chunk list), 256 tokens chunks of 64 (one launch per
+    ring step)."""
     import picotron_amd.process_group_manager as pgm
     from picotron_amd.context_parallel import context_parallel as cp
     from picotron_amd.model import Llama
-    cfg = OM.LlamaShape(256, 4, 2, 512, 1024, 2, 256)
-    ids, tgt = OM.synthetic_batch(cfg.vocab_size, 2, 256, seed=1)
+    monkeypatch.setenv("PICO_FUSED_ROPE", fused_rope)
+    cfg = OM.LlamaShape(256, 4, 2, 512, 1024, 2, seq)
+    ids, tgt = OM.synthetic_batch(cfg.vocab_size, 2, seq, seed=1)
     ids, tgt = ids.to(device), tgt.to(device)
 
     torch.manual_seed(0)
@@ -293,11 +312,11 @@ def test_model_cp4_virtual_ranks_equals_cp1(pgm1, device):
     m4 = Llama(cfg).to(torch.bfloat16).to(device)
     cp.apply_context_parallel(m4)
     assert os.environ["CONTEXT_PARALLEL"] == "1"
-    per = 256 // W
+    per = seq // W
     total = 0.0
     for r in range(W):
         m4.set_cp_rank(r)
-        pos = OR.position_ids(r, 256, W, 2)
+        pos = OR.position_ids(r, seq, W, 2)
         assert pos[0, 0].item() == r * per
         logits = m4(ids[:, r * per:(r + 1) * per])
         # each rank's mean CE; the reference averages the ranks' losses (utils.py:94-99)

@@ -1,6 +1,6 @@
 """Host logic of the virtual-rank ring (RingAttentionFunc, LocalRing, ContextCommunicate) on the CPU.
 
-The four kernel wrappers the ring calls are replaced by fp32 torch stand-ins (block maths written out below), so that
+The kernel wrappers the ring calls are replaced by fp32 torch stand-ins (block maths written out below), so that
 what is under test is the schedule, the mailbox and the accumulation of dK / dV across ranks -- checked against
 full-sequence attention differentiated by autograd, which knows nothing of chunks or rings.  The GPU tests run the
 same scenarios on the HIP kernels.
@@ -79,8 +79,56 @@ def fake_convert_f32(src, dtype, like=None, bshd=False, strides=None):
     return src.to(dtype)
 
 
-@pytest.fixture()
-def ring(monkeypatch):
+def _full_scores(q, k_all, sm_scale, causal, q_offset):
+    s = q @ k_all.transpose(-1, -2) * sm_scale
+    if causal:
+        qi = torch.arange(q.size(2)).unsqueeze(1) + q_offset
+        kj = torch.arange(k_all.size(2)).unsqueeze(0)
+        s = s.masked_fill(kj > qi, float("-inf"))
+    return s
+
+
+def fake_attn_fwd_chunks(q, ks, vs, sm_scale, causal, q_offset=0, out=None, lse=None, merge=False, out_dtype=torch.bfloat16,
+                         bshd_out=False, rope=None, q_pos_offset=0, want_q_rot=False):
+    """All listed chunks in one go: softmax over their concatenation, query i at position q_offset + i."""
+    assert rope is None and not merge
+    qf, kf, vf, _ = _expand(q, torch.cat(ks, 2), torch.cat(vs, 2))
+    s = _full_scores(qf, kf, sm_scale, causal, q_offset)
+    return (torch.softmax(s, -1) @ vf).to(out_dtype), torch.logsumexp(s, -1), None
+
+
+def fake_attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale, causal, q_offset=0, dq=None, dks=None, dvs=None, dq_accumulate=False,
+                         dkv_accumulate=None, out=None, delta=None, rope=None, q_pos_offset=0, k_pos_offset=0):
+    assert rope is None
+    Sc = ks[0].size(2)
+    qf, kf, vf, rep = _expand(q, torch.cat(ks, 2), torch.cat(vs, 2))
+    do = dout.float()
+    if delta is None:
+        delta = (do * out.float()).sum(-1)
+    p = torch.exp(_full_scores(qf, kf, sm_scale, causal, q_offset) - lse.unsqueeze(-1))
+    ds = p * (do @ vf.transpose(-1, -2) - delta.unsqueeze(-1))
+    b_dv = _fold(p.transpose(-1, -2) @ do, rep)
+    b_dk = _fold(ds.transpose(-1, -2) @ qf * sm_scale, rep)
+    if dq is not None:
+        b_dq = ds @ kf * sm_scale
+        dq.add_(b_dq) if dq_accumulate else dq.copy_(b_dq)
+    for c in range(len(ks)):
+        if dks is None or dks[c] is None:
+            continue
+        sl = slice(c * Sc, (c + 1) * Sc)
+        if dkv_accumulate is not None and dkv_accumulate[c]:
+            dks[c].add_(b_dk[:, :, sl])
+            dvs[c].add_(b_dv[:, :, sl])
+        else:
+            dks[c].copy_(b_dk[:, :, sl])
+            dvs[c].copy_(b_dv[:, :, sl])
+    return delta
+
+
+@pytest.fixture(params=["one_launch_per_rank", "one_launch_per_ring_step"])
+def ring(monkeypatch, request):
+    """Both shapes of the ring: all steps of a rank in one call over the chunk list (the default when the chunks fit
+    one launch; the stand-in says they do) and the reference's one call per ring step with hops between."""
     import picotron_amd.process_group_manager as pgm
     from picotron_amd import ops
     from picotron_amd.context_parallel import context_parallel as cp
@@ -88,6 +136,9 @@ def ring(monkeypatch):
     monkeypatch.setattr(ops, "attn_bwd", fake_attn_bwd)
     monkeypatch.setattr(ops, "attn_bwd_preprocess", fake_attn_bwd_preprocess)
     monkeypatch.setattr(ops, "convert_f32", fake_convert_f32)
+    monkeypatch.setattr(ops, "attn_fwd_chunks", fake_attn_fwd_chunks)
+    monkeypatch.setattr(ops, "attn_bwd_chunks", fake_attn_bwd_chunks)
+    monkeypatch.setattr(ops, "chunks_fit_one_launch", lambda ks, vs: request.param == "one_launch_per_rank")
     yield pgm, cp
     pgm.setup_process_group_manager(1, 1, 1, 1)
 
