@@ -230,6 +230,9 @@ def ring_api_extra(torch, ops, rb, iters=20):
     total_flops = sum(rb.flops())
 
     def step():
+        # a new pass: the same leaf tensors come back every step, and without this the mailbox would take them for
+        # chunks staged ahead and hand out the previous step's publishing nodes
+        mgr.cp_ring.reset()
         outs = []
         for r in range(W):
             mgr.set_cp_rank(r)

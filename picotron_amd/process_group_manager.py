@@ -68,7 +68,10 @@ class LocalRing:
     def reset(self) -> None:
         """Forget every published chunk.  The mailbox keeps the last pass's K / V alive until the next pass begins
         (a later rank, or a rank's forward that follows another rank's backward, may still read them); call this to
-        free them earlier."""
+        free them earlier.  A loop that feeds the SAME k / v tensor objects to every pass (a benchmark, a step that is
+        recorded into a HIP graph after warm-up passes) must call it at the start of each pass: unchanged tensors are
+        otherwise taken for chunks staged ahead of the play, and the pass would reuse the previous pass's autograd
+        nodes (harmless in eager runs, but a recorded graph would miss their work)."""
         self.chunks.clear()
         self._next_slot = 0
 
