@@ -10,23 +10,11 @@ namespace {
 
 constexpr int kThreads = 512;
 constexpr int kWaves = kThreads / kWave;
-// streaming switches (the logits of a training step are far larger than the caches): forward loads +13 %, backward
-// loads and stores together +6 % at [4096, 49152]
-#ifndef PICO_NT_CE_FWD_LOADS
-#define PICO_NT_CE_FWD_LOADS 1
-#endif
-#ifndef PICO_NT_CE_BWD_LOADS
-#define PICO_NT_CE_BWD_LOADS 1
-#endif
-#ifndef PICO_CE_BWD_UNROLL
-#define PICO_CE_BWD_UNROLL 4
-#endif
-#ifndef PICO_CE_FWD_UNROLL
-#define PICO_CE_FWD_UNROLL 2
-#endif
-#ifndef PICO_NT_CE_BWD_STORES
-#define PICO_NT_CE_BWD_STORES 1
-#endif
+// The logits of a training step are far larger than the caches, so they are read with streaming loads and dlogits
+// leave with streaming stores (forward +13 %, backward +6 % at [4096, 49152]); a thread requests several pieces of its
+// row before it uses the first (bytes in flight per thread: forward 2, backward 4 pieces).
+constexpr bool kStreamLoads = true, kStreamStores = true;
+constexpr int kFwdUnroll = 2, kBwdUnroll = 4;
 
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
@@ -54,18 +42,18 @@ __global__ __launch_bounds__(kThreads) void ce_fwd_kernel(const T* __restrict__ 
 #pragma unroll
     for (int i = 0; i < V; ++i) s += fast_exp2(e[i] * kLog2e - m);
   };
-  constexpr int U = PICO_CE_FWD_UNROLL;   // pieces of the row requested together (bytes in flight per thread)
+  constexpr int U = kFwdUnroll;   // pieces of the row requested together (bytes in flight per thread)
   int v = threadIdx.x;
   for (; v + (U - 1) * kThreads < nvec; v += U * kThreads) {
     float e[U][V];
 #pragma unroll
-    for (int u = 0; u < U; ++u) load_as<T, PICO_NT_CE_FWD_LOADS != 0>(x + static_cast<int64_t>(v + u * kThreads) * V, e[u]);
+    for (int u = 0; u < U; ++u) load_as<T, kStreamLoads>(x + static_cast<int64_t>(v + u * kThreads) * V, e[u]);
 #pragma unroll
     for (int u = 0; u < U; ++u) absorb(e[u]);
   }
   for (; v < nvec; v += kThreads) {
     float e[V];
-    load_as<T, PICO_NT_CE_FWD_LOADS != 0>(x + static_cast<int64_t>(v) * V, e);
+    load_as<T, kStreamLoads>(x + static_cast<int64_t>(v) * V, e);
     absorb(e);
   }
   for (int j = nvec * V + threadIdx.x; j < vocab; j += kThreads) {  // tail when vocab is not a multiple of V
@@ -109,12 +97,12 @@ __global__ __launch_bounds__(kThreads) void ce_bwd_kernel(const T* __restrict__ 
   const int nvec = vocab / V;
   // kCeUnroll pieces of the row per thread are requested before the first is used: one 16-byte load per thread at a
   // time leaves too few bytes in flight to cover the memory latency
-  constexpr int U = PICO_CE_BWD_UNROLL;
+  constexpr int U = kBwdUnroll;
   int v = threadIdx.x;
   for (; v + (U - 1) * kThreads < nvec; v += U * kThreads) {
     float e[U][V];
 #pragma unroll
-    for (int u = 0; u < U; ++u) load_as<T, PICO_NT_CE_BWD_LOADS != 0>(x + static_cast<int64_t>(v + u * kThreads) * V, e[u]);
+    for (int u = 0; u < U; ++u) load_as<T, kStreamLoads>(x + static_cast<int64_t>(v + u * kThreads) * V, e[u]);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       float o[V];
@@ -124,19 +112,19 @@ __global__ __launch_bounds__(kThreads) void ce_bwd_kernel(const T* __restrict__ 
         const float p = fast_exp2(e[u][i] * kLog2e - l2);
         o[i] = (p - ((j0 + i) == t ? 1.f : 0.f)) * scale;
       }
-      store_as<T, PICO_NT_CE_BWD_STORES != 0>(d + static_cast<int64_t>(v + u * kThreads) * V, o);
+      store_as<T, kStreamStores>(d + static_cast<int64_t>(v + u * kThreads) * V, o);
     }
   }
   for (; v < nvec; v += kThreads) {
     float e[V], o[V];
-    load_as<T, PICO_NT_CE_BWD_LOADS != 0>(x + static_cast<int64_t>(v) * V, e);
+    load_as<T, kStreamLoads>(x + static_cast<int64_t>(v) * V, e);
     const int j0 = v * V;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       const float p = fast_exp2(e[i] * kLog2e - l2);
       o[i] = (p - ((j0 + i) == t ? 1.f : 0.f)) * scale;
     }
-    store_as<T, PICO_NT_CE_BWD_STORES != 0>(d + static_cast<int64_t>(v) * V, o);
+    store_as<T, kStreamStores>(d + static_cast<int64_t>(v) * V, o);
   }
   for (int j = nvec * V + threadIdx.x; j < vocab; j += kThreads) {
     const float p = fast_exp2(static_cast<float>(x[j]) * kLog2e - l2);

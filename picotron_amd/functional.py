@@ -1,6 +1,8 @@
 """autograd.Functions that tie the HIP forward and backward kernels together for the model code."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from . import ops
@@ -99,6 +101,14 @@ class CrossEntropyFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, logits, targets, ignore_index=-100):
+        if os.getenv("PICO_CHECK_TARGETS", "0") == "1":
+            # F.cross_entropy asserts on the device for a target outside [0, vocab) (train.py:46-49); the kernels skip such
+            # a row instead (they may not index with it), which would hide a tokenizer / vocabulary mismatch.  This
+            # opt-in check costs a host synchronisation.
+            bad = (targets != ignore_index) & ((targets < 0) | (targets >= logits.size(-1)))
+            if bool(bad.any()):
+                raise RuntimeError(f"cross_entropy: {int(bad.sum())} targets lie outside [0, {logits.size(-1)}) and are not "
+                                   f"ignore_index={ignore_index}")
         loss_rows, lse = ops.cross_entropy_fwd(logits, targets, ignore_index)
         # rows that count: not ignored and a valid index (the kernels skip a target outside [0, vocab) as well)
         count = ((targets != ignore_index) & (targets >= 0) & (targets < logits.size(-1))).sum().clamp(min=1).to(torch.float32)
@@ -145,7 +155,6 @@ class FusedLinearFunc(torch.autograd.Function):
 
 def _fused_rope() -> bool:
     """RoPE inside the attention kernels (default); PICO_FUSED_ROPE=0 keeps it a launch of its own over q and k."""
-    import os
     return os.getenv("PICO_FUSED_ROPE", "1") != "0"
 
 

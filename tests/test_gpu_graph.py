@@ -4,6 +4,7 @@ The entry points only enqueue kernels on the stream they are given (no allocatio
 nodes), so a caller may record a whole layer into one graph.  The graph is replayed several times with the program's
 own eager work and synchronisations in between, and every replay is compared bit for bit with the eager results (the
 kernels are deterministic: no atomics)."""
+import ctypes
 import math
 
 import pytest
@@ -19,8 +20,9 @@ def rnd(*shape, seed=0, scale=1.0):
 
 @pytest.mark.parametrize("D,Hq,Hkv,S", [(64, 8, 8, 640), (128, 8, 2, 1100)])
 def test_layer_sized_call_sequence_replays_like_eager_launches(device, D, Hq, Hkv, S):
-    from picotron_amd import ops
+    from picotron_amd import _lib, ops
     from picotron_amd.model import get_cos_sin
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
     B, hidden, inter, vocab = 2, 512, 1024, 3000
     rows = B * S
     scale = 1 / math.sqrt(D)
@@ -61,6 +63,13 @@ def test_layer_sized_call_sequence_replays_like_eager_launches(device, D, Hq, Hk
         y, rstd, res_out = ops.rmsnorm_fwd(x, w, 1e-5, False, residual=res, want_residual_out=True)
         dx, dw = ops.rmsnorm_bwd(dy, res_out, w, rstd, dresidual=dy, dw_dtype=bf)
         r.update(y=y, rstd=rstd, res_out=res_out, dx=dx, dw=dw)
+        # the entry point that allocates nothing (its first call on a device, which looks up the address of its static
+        # array, was made by the eager run above: that call must lie outside a capture)
+        dx_s, dw_s = torch.empty_like(dx), torch.empty_like(dw)
+        _lib.check(_lib.lib().pico_rmsnorm_bwd_static(
+            P(dy), P(res_out), P(w), P(rstd), P(dy), P(dx_s), P(dw_s), _lib.PICO_BF16, rows, hidden, _lib.PICO_BF16,
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        r.update(dx_s=dx_s, dw_s=dw_s)
         # SwiGLU on the halves of one projection output
         gate, up = gate_up[:, :inter], gate_up[:, inter:]
         hmid = ops.swiglu_fwd(gate, up)

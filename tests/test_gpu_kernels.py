@@ -698,6 +698,14 @@ def test_cross_entropy_target_out_of_range_is_skipped_not_read(ops, device):
         assert loss_rows[r].item() == 0.0 and xd.grad[r].abs().max().item() == 0.0
     gw = OL.cross_entropy_backward(x[keep], t[keep], 1.0)
     assert maxabs(xd.grad[keep.to(device)], gw) <= 2 ** -8 * gw.abs().max().item() + 1e-9
+    # and with the opt-in host check the same input is an error, as it is for F.cross_entropy (train.py:46-49)
+    import os
+    os.environ["PICO_CHECK_TARGETS"] = "1"
+    try:
+        with pytest.raises(RuntimeError, match="outside"):
+            cross_entropy(xd, t.to(device), -1)
+    finally:
+        os.environ.pop("PICO_CHECK_TARGETS", None)
 
 
 def test_fused_adamw_overlapped_with_backward_gives_the_same_update(device):
