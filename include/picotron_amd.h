@@ -256,6 +256,11 @@ int pico_attn_bwd_rope(const pico_attn_desc* desc, const void* q_rot, const void
  * merge pass, no fp32 running out.
  * Backward: dk[c] / dv[c] receive chunk c's gradient; a NULL pair means that chunk's gradient is not wanted; bit c of
  * accumulate_mask adds to what is there (fp32 only: the chunk's travelling accumulators).
+ * dk_final[c] / dv_final[c] (optional, given together): this launch holds the LAST block that chunk c's gradient is
+ * waiting for (context_parallel.py:104-110: the accumulators have come round the ring).  The chunk's total -- what
+ * dk[c] / dv[c] hold, if bit c of accumulate_mask is set, plus this launch's block -- is then rounded once and written
+ * to dk_final[c] / dv_final[c] in bf16, addressed by final_stride (element strides b, h, s); dk[c] / dv[c] are only
+ * read.  It saves the fp32 write, the read-back and the separate cast.
  */
 #define PICO_MAX_KV_CHUNKS 16
 typedef struct pico_kv_chunks {
@@ -265,6 +270,9 @@ typedef struct pico_kv_chunks {
   const void* v[PICO_MAX_KV_CHUNKS];
   void* dk[PICO_MAX_KV_CHUNKS];        /* backward only */
   void* dv[PICO_MAX_KV_CHUNKS];
+  void* dk_final[PICO_MAX_KV_CHUNKS];  /* backward only, optional */
+  void* dv_final[PICO_MAX_KV_CHUNKS];
+  int64_t final_stride[3];
   uint32_t accumulate_mask;
   uint32_t reserved;
 } pico_kv_chunks;

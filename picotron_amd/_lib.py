@@ -35,8 +35,9 @@ MAX_KV_CHUNKS = 16
 class KvChunks(Structure):
     """Mirror of ``pico_kv_chunks``."""
     _fields_ = [("count", c_int32), ("chunk_len", c_int32), ("k", c_void_p * MAX_KV_CHUNKS), ("v", c_void_p * MAX_KV_CHUNKS),
-                ("dk", c_void_p * MAX_KV_CHUNKS), ("dv", c_void_p * MAX_KV_CHUNKS), ("accumulate_mask", ctypes.c_uint32),
-                ("reserved", ctypes.c_uint32)]
+                ("dk", c_void_p * MAX_KV_CHUNKS), ("dv", c_void_p * MAX_KV_CHUNKS),
+                ("dk_final", c_void_p * MAX_KV_CHUNKS), ("dv_final", c_void_p * MAX_KV_CHUNKS), ("final_stride", c_int64 * 3),
+                ("accumulate_mask", ctypes.c_uint32), ("reserved", ctypes.c_uint32)]
 
 
 _P = c_void_p

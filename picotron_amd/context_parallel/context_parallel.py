@@ -72,6 +72,7 @@ class _PublishKV(torch.autograd.Function):
         ctx.set_materialize_grads(False)
         # layout only, no saved tensors: the node may run in several backward calls (one rank's loss at a time)
         ctx.layout = tuple((t.dtype, t.stride() if ops._dense(t) and t.stride(-1) == 1 else None) for t in (k, v))
+        box.layout = ctx.layout
         if rope is not None:
             cos, sin, pos0 = rope
             return ops.rope(k, cos, sin, pos_offset=pos0), v.view_as(v)
@@ -81,7 +82,12 @@ class _PublishKV(torch.autograd.Function):
     def backward(ctx, gk, gv):
         box = ctx.box
         dk = dv = None
-        if box.dk is not None:
+        box.arrived = 0
+        if box.final_dk is not None:
+            # the last reader's kernel wrote the rounded totals itself
+            dk, dv = box.final_dk, box.final_dv
+            box.final_dk = box.final_dv = box.dk = box.dv = None
+        elif box.dk is not None:
             (k_dtype, k_strides), (v_dtype, v_strides) = ctx.layout
             dk = ops.convert_f32(box.dk, k_dtype, strides=k_strides)
             dv = ops.convert_f32(box.dv, v_dtype, strides=v_strides)
@@ -138,6 +144,10 @@ class RingAttentionFunc(torch.autograd.Function):
                 chunks[held] = ring.fetch(slot, held, rank)
         peers = [c for c in sorted(chunks) if c != rank]
         flat = [t for c in peers for t in (chunks[c].k, chunks[c].v)]
+        if torch.is_grad_enabled():
+            for c in chunks.values():
+                if c.k.requires_grad or c.v.requires_grad:
+                    c.grads.readers += 1
         return super().apply(q, own.k, own.v, sm_scale, is_causal, (slot, rank, world, chunks, peers), table, *flat)
 
     @staticmethod
@@ -233,18 +243,41 @@ class RingAttentionFunc(torch.autograd.Function):
                 box.dv = torch.empty(shape, dtype=torch.float32, device=q.device)
             return box.dk, box.dv, not fresh
 
+        def finals(c):
+            """bf16 buffers for chunk c's totals if this rank's block is the last one they wait for (every rank that
+            read the chunk has added its block), in the chunk's own layout; else None."""
+            box = chunks[c].grads
+            box.arrived += 1
+            (k_dtype, k_strides), (v_dtype, v_strides) = box.layout if box.layout is not None else ((None, None), (None, None))
+            if box.arrived != box.readers or k_dtype not in ops.FINAL_TOTAL_DTYPES or v_dtype != k_dtype:
+                return None
+            shape = chunks[c].k.shape
+            if k_strides is not None and k_strides == v_strides:
+                box.final_dk = torch.empty_strided(shape, k_strides, dtype=k_dtype, device=q.device)
+                box.final_dv = torch.empty_strided(shape, k_strides, dtype=k_dtype, device=q.device)
+            else:   # chunks that are views with gaps (or k and v laid out differently): contiguous gradients
+                box.final_dk = torch.empty(shape, dtype=k_dtype, device=q.device)
+                box.final_dv = torch.empty(shape, dtype=k_dtype, device=q.device)
+            return box.final_dk, box.final_dv
+
         if ctx.one_launch is not None:
             order, q_off = ctx.one_launch
             ks = [chunks[c].k.detach() for c in order]
             vs = [chunks[c].v.detach() for c in order]
-            got = [boxes(c) if wants[c] else (None, None, False) for c in order]
+            fin = {c: finals(c) if wants[c] else None for c in order}
+            # a chunk whose totals leave from this launch needs fp32 sums only if earlier blocks left some
+            got = [(None, None, False) if not wants[c] else
+                   ((chunks[c].grads.dk, chunks[c].grads.dv, chunks[c].grads.dk is not None) if fin[c] is not None else boxes(c))
+                   for c in order]
             dq = None
             if ctx.needs_input_grad[0]:
                 dq = (torch.empty_strided(q.shape, q.stride(), dtype=q.dtype, device=q.device)
                       if ops._dense(q) and q.stride(-1) == 1 else torch.empty(q.shape, dtype=q.dtype, device=q.device))
             ops.attn_bwd_chunks(dout, q, ks, vs, softmax_lse, sm_scale, is_causal, q_off, dq, [g[0] for g in got],
                                 [g[1] for g in got], dkv_accumulate=[g[2] for g in got], out=out, rope=cs,
-                                q_pos_offset=q_pos, k_pos_offset=q_pos - q_off if is_causal else 0)
+                                q_pos_offset=q_pos, k_pos_offset=q_pos - q_off if is_causal else 0,
+                                dk_finals=[fin[c][0] if fin[c] is not None else None for c in order],
+                                dv_finals=[fin[c][1] if fin[c] is not None else None for c in order])
             return (dq,) + nothing[1:]
 
         delta = ops.attn_bwd_preprocess(dout, out)

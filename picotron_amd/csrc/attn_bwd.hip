@@ -32,6 +32,9 @@ struct BwdParams {
   void* dq;
   void* dk[kMaxChunks];      // per K / V chunk; nullptr: that chunk's gradient is not wanted
   void* dv[kMaxChunks];
+  __bf16* dk_final[kMaxChunks];   // per chunk, optional: the chunk's total (fp32 dk[c] if its accumulate bit is set, plus this
+  __bf16* dv_final[kMaxChunks];   //   launch's block) leaves here in bf16; dk[c] / dv[c] are only read
+  int64_t dkfs[3];                // element strides (b, h, s) of dk_final / dv_final
   uint32_t dkv_accumulate;   // bit c: chunk c's dk / dv are added to (fp32)
   int dq_f32, dq_accumulate;
   int dkv_f32;
@@ -96,7 +99,7 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
   const int key0 = ktile * BN;                     // position of the tile's first key in the launch
   const int chunk = a.kv.count > 1 ? key0 / a.kv.len : 0;
   const int crow0 = key0 - chunk * a.kv.len;       // ... and its row in the chunk that holds it
-  if (p.dk[chunk] == nullptr) return;              // this chunk's gradient is not wanted (uniform over the workgroup)
+  if (p.dk[chunk] == nullptr && p.dk_final[chunk] == nullptr) return;   // this chunk's gradient is not wanted (uniform over the workgroup)
   const int tid = threadIdx.x, wave_id = tid / 64, lane = tid % 64;
   // wave: which 32 keys of the tile; pair_sb (PAIR only): which 32-query sub-block of every query tile
   const int wave = PAIR ? __builtin_amdgcn_readfirstlane(wave_id % C::kKeyWaves) : wave_id;
@@ -542,7 +545,14 @@ __device__ __forceinline__ void attn_bwd_dkdv_tile(const BwdParams& p, const int
     // gradient w.r.t. the un-rotated k: rotate the lane's row of dK back (linear, so the scale and the sum can follow)
     if (p.rope.cos != nullptr) rope_unrotate_acc<D>(dk_acc, p.rope, n < rows_live ? p.rope.k_pos0 + kw0 + n : 0, h);
     const bool accumulate = (p.dkv_accumulate >> chunk) & 1u;
-    if (p.dkv_f32) {
+    if (p.dk_final[chunk] != nullptr) {
+      // the last block this chunk's gradient was waiting for: total = travelling sums + this block, rounded once
+      const int64_t foff = b * p.dkfs[0] + hkv * p.dkfs[1] + static_cast<int64_t>(row0) * p.dkfs[2];
+      wave_store_rows_total<D>(region, dk_acc, a.sm_scale, accumulate ? static_cast<const float*>(p.dk[chunk]) + off : nullptr, p.dks[2],
+                               p.dk_final[chunk] + foff, p.dkfs[2], rows_live, lane);
+      wave_store_rows_total<D>(region, dv_acc, 1.f, accumulate ? static_cast<const float*>(p.dv[chunk]) + off : nullptr, p.dks[2],
+                               p.dv_final[chunk] + foff, p.dkfs[2], rows_live, lane);
+    } else if (p.dkv_f32) {
       wave_store_rows<D, true>(region, dk_acc, a.sm_scale, static_cast<float*>(p.dk[chunk]) + off, p.dks[2], rows_live, lane, accumulate, false);
       wave_store_rows<D, true>(region, dv_acc, 1.f, static_cast<float*>(p.dv[chunk]) + off, p.dks[2], rows_live, lane, accumulate, false);
     } else {
@@ -961,16 +971,33 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const pic
   // a gradient that is not wanted is passed as NULL and its kernel (or its chunk's workgroups) is skipped
   bool want_dkv = false;
   p.dkv_accumulate = 0;
-  for (int c = 0; c < kMaxChunks; ++c) p.dk[c] = p.dv[c] = nullptr;
+  for (int c = 0; c < kMaxChunks; ++c) {
+    p.dk[c] = p.dv[c] = nullptr;
+    p.dk_final[c] = p.dv_final[c] = nullptr;
+  }
+  bool any_final = false;
   for (int c = 0; c < kv->count; ++c) {
-    if ((kv->dk[c] == nullptr) != (kv->dv[c] == nullptr))
-      return fail(PICO_ERR_NULL, "%s: dk and dv must be given together (chunk %d)", fn, c);
+    if ((kv->dk[c] == nullptr) != (kv->dv[c] == nullptr) || (kv->dk_final[c] == nullptr) != (kv->dv_final[c] == nullptr))
+      return fail(PICO_ERR_NULL, "%s: dk and dv (and dk_final and dv_final) must be given together (chunk %d)", fn, c);
+    if (!aligned16(kv->dk_final[c]) || !aligned16(kv->dv_final[c]))
+      return fail(PICO_ERR_ALIGN, "%s: chunk %d: dk_final and dv_final must be 16-byte aligned", fn, c);
     p.dk[c] = kv->dk[c];
     p.dv[c] = kv->dv[c];
-    if (kv->dk[c]) {
-      want_dkv = true;
-      if ((kv->accumulate_mask >> c) & 1u) p.dkv_accumulate |= 1u << c;
+    p.dk_final[c] = static_cast<__bf16*>(kv->dk_final[c]);
+    p.dv_final[c] = static_cast<__bf16*>(kv->dv_final[c]);
+    const bool acc = kv->dk[c] && ((kv->accumulate_mask >> c) & 1u);
+    if (kv->dk[c] || kv->dk_final[c]) want_dkv = true;
+    if (acc) p.dkv_accumulate |= 1u << c;
+    if (kv->dk_final[c]) {
+      any_final = true;
+      if (acc && dkv_dtype != PICO_F32)
+        return fail(PICO_ERR_DTYPE, "%s: chunk %d: the sums that dk_final completes must be fp32", fn, c);
     }
+  }
+  for (int i = 0; i < 3; ++i) {
+    p.dkfs[i] = any_final ? kv->final_stride[i] : 0;
+    if (any_final && (p.dkfs[i] < 0 || p.dkfs[i] % 4 != 0))
+      return fail(PICO_ERR_STRIDE, "%s: final_stride must hold non-negative multiples of 4 elements", fn);
   }
   if (p.dkv_accumulate && dkv_dtype != PICO_F32) return fail(PICO_ERR_DTYPE, "%s: accumulate needs fp32 gradients", fn);
   const bool want_dq = dq != nullptr;

@@ -191,6 +191,49 @@ __device__ __forceinline__ void wave_store_rows(unsigned char* region, const f32
   }
 }
 
+// The same rows as the sum of an fp32 buffer and the accumulators, rounded once to bf16 and written somewhere else:
+// the last block of a ring adds itself to the travelling fp32 sums (`old_row0`, nullptr: nothing to add) and hands
+// the total back in the dtype of the inputs.  32 columns per pass (fp32 staging), 8-byte bf16 pieces per lane.
+template <int D>
+__device__ __forceinline__ void wave_store_rows_total(unsigned char* region, const f32x16 (&acc)[D / 32], float scale,
+                                                      const float* old_row0, int64_t old_stride, __bf16* dst_row0,
+                                                      int64_t dst_stride, int rows_live, int lane) {
+  constexpr int kPitch = 144;
+  const int n = lane % 32, h = lane / 32;
+#pragma unroll
+  for (int c0 = 0; c0 < D; c0 += 32) {
+    const int db = c0 / 32;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      f32x4 v4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) v4[t] = acc[db][4 * j + t] * scale;
+      *reinterpret_cast<f32x4*>(region + n * kPitch + (8 * j + 4 * h) * 4) = v4;
+    }
+    f32x4 v[4], old[4];
+    int row[4], piece[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int idx = lane + 64 * t;
+      row[t] = idx / 8;
+      piece[t] = idx % 8;
+      v[t] = *reinterpret_cast<const f32x4*>(region + row[t] * kPitch + piece[t] * 16);
+      old[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (old_row0 != nullptr && row[t] < rows_live)
+        old[t] = *reinterpret_cast<const f32x4*>(old_row0 + static_cast<int64_t>(row[t]) * old_stride + c0 + piece[t] * 4);
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      if (row[t] < rows_live) {
+        bf16x4 o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = static_cast<__bf16>(v[t][e] + old[t][e]);
+        __builtin_nontemporal_store(__builtin_bit_cast(u32x2, o),
+                                    reinterpret_cast<u32x2*>(dst_row0 + static_cast<int64_t>(row[t]) * dst_stride + c0 + piece[t] * 4));
+      }
+  }
+}
+
 // ---- RoPE inside the attention kernels (non-interleaved: column d pairs with d + D/2; model.py:12-19).
 // Tables are [rows, >= D/2 columns] with `pitch` elements between rows, bf16 or fp32; row index = position.
 struct RopeArgs {

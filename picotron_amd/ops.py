@@ -306,6 +306,9 @@ def attn_bwd_rope(dout, q_rot, k_rot, v, out, lse, cos, sin, sm_scale: float, ca
 
 
 # ---- all ring steps of one rank in one launch: K / V as a list of equally shaped chunk tensors
+FINAL_TOTAL_DTYPES = (torch.bfloat16,)   # dtypes attn_bwd_chunks can write a chunk's rounded totals in (dk_finals / dv_finals)
+
+
 def chunks_fit_one_launch(ks, vs) -> bool:
     """True if the chunk tensors can go to the chunk-list entry points as they are: at most 16 bf16 chunks of one shape
     and one stride triple (k's may differ from v's), unit D stride, strides that are multiples of 8, and -- with several
@@ -324,7 +327,7 @@ def chunks_fit_one_launch(ks, vs) -> bool:
     return True
 
 
-def _kv_chunks(ks, vs, dks=None, dvs=None, accumulate=None) -> KvChunks:
+def _kv_chunks(ks, vs, dks=None, dvs=None, accumulate=None, dk_finals=None, dv_finals=None) -> KvChunks:
     c = KvChunks()
     c.count, c.chunk_len = len(ks), ks[0].size(2)
     mask = 0
@@ -334,6 +337,9 @@ def _kv_chunks(ks, vs, dks=None, dvs=None, accumulate=None) -> KvChunks:
             c.dk[i], c.dv[i] = dks[i].data_ptr(), dvs[i].data_ptr()
             if accumulate is not None and accumulate[i]:
                 mask |= 1 << i
+        if dk_finals is not None and dk_finals[i] is not None:
+            c.dk_final[i], c.dv_final[i] = dk_finals[i].data_ptr(), dv_finals[i].data_ptr()
+            c.final_stride[0], c.final_stride[1], c.final_stride[2] = dk_finals[i].stride()[:3]
     c.accumulate_mask = mask
     return c
 
@@ -380,11 +386,14 @@ def attn_fwd_chunks(q, ks, vs, sm_scale: float, causal: bool, q_offset: int = 0,
 
 def attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale: float, causal: bool, q_offset: int = 0, dq=None, dks=None, dvs=None,
                     dq_accumulate: bool = False, dkv_accumulate=None, out=None, delta=None, rope=None,
-                    q_pos_offset: int = 0, k_pos_offset: int = 0):
+                    q_pos_offset: int = 0, k_pos_offset: int = 0, dk_finals=None, dv_finals=None):
     """attn_bwd over a chunk list.  dks / dvs: per chunk a gradient buffer (all of one dtype and stride triple) or None
     (not wanted); dkv_accumulate: per chunk, add to the fp32 buffer instead of writing it.  dq None: not wanted.  With
     `out` (forward output) delta is computed inside the call, otherwise `delta` must be given.  rope = (cos, sin): q and
-    the chunks' k are rotated tensors, dq / dk leave un-rotated.  Returns delta."""
+    the chunks' k are rotated tensors, dq / dk leave un-rotated.  dk_finals / dv_finals: per chunk a bf16 buffer (all of
+    one stride triple) or None; where given, this call holds the last block the chunk's gradient waits for, and the
+    total -- the fp32 sums in dks / dvs (if the chunk's dkv_accumulate flag is set) plus this block -- is written there,
+    rounded once; the fp32 buffers are only read.  Returns delta."""
     _dev(dout, q, lse, dq, out, delta)
     if not chunks_fit_one_launch(ks, vs):
         raise RuntimeError("attn_bwd_chunks: the chunks do not fit one launch (see chunks_fit_one_launch)")
@@ -413,8 +422,19 @@ def attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale: float, causal: bool, q_offse
     if dq is not None and dq.stride(-1) != 1:
         raise RuntimeError("attn_bwd_chunks: dq needs a unit D stride")
     dqs = (ctypes.c_int64 * 3)(*(dq.stride()[:3] if dq is not None else (0, 0, 0)))
+    finals = [t for t in (dk_finals or []) if t is not None]
+    if finals:
+        f0 = finals[0]
+        for a, b_ in zip(dk_finals, dv_finals):
+            if (a is None) != (b_ is None):
+                raise RuntimeError("attn_bwd_chunks: dk_final and dv_final of a chunk must be given together")
+            if a is not None and (a.dtype != torch.bfloat16 or b_.dtype != torch.bfloat16 or a.stride() != f0.stride()
+                                  or b_.stride() != f0.stride() or a.stride(-1) != 1 or a.shape != ks[0].shape
+                                  or not a.is_cuda or not b_.is_cuda):
+                raise RuntimeError("attn_bwd_chunks: dk_final / dv_final must be bf16 buffers of the chunks' shape that share "
+                                   "one stride triple (unit D stride)")
     d = _chunk_desc(q, ks, vs, dout, sm_scale, causal, q_offset)
-    kv = _kv_chunks(ks, vs, dks if given else None, dvs, dkv_accumulate)
+    kv = _kv_chunks(ks, vs, dks if given else None, dvs, dkv_accumulate, dk_finals if finals else None, dv_finals)
     tables = ctypes.byref(_rope_tables(*rope)) if rope is not None else None
     check(_lib.lib().pico_attn_bwd_chunks(ctypes.byref(d), _ptr(q), ctypes.byref(kv), _ptr(dout), _ptr(out),
                                           _dt(out, "out") if out is not None else PICO_BF16, _ptr(lse.contiguous()), _ptr(delta),

@@ -19,11 +19,18 @@ class GradBox:
     (``context_parallel.py:85-106``).  Every rank's backward adds its block here; the chunk's own autograd node
     hands the total back once all of them have run."""
 
-    __slots__ = ("dk", "dv")
+    __slots__ = ("dk", "dv", "readers", "arrived", "final_dk", "final_dv", "layout")
 
     def __init__(self):
         self.dk: Optional[torch.Tensor] = None
         self.dv: Optional[torch.Tensor] = None
+        self.readers = 0        # ranks whose forward read the chunk and will add a block in their backward
+        self.arrived = 0        # ... and how many of them have done so since the sums were last handed back
+        # the block that completes the sums is written rounded, in the chunk's own dtype and layout, by the kernel
+        # that computes it (one pass less than fp32 sums + a cast); `layout` = ((k dtype, strides), (v dtype, strides))
+        self.final_dk: Optional[torch.Tensor] = None
+        self.final_dv: Optional[torch.Tensor] = None
+        self.layout = None
 
 
 class RingChunk:

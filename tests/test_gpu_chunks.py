@@ -97,6 +97,19 @@ def test_chunk_list_equals_contiguous_keys_and_oracle(ops, device, B, Hq, Hkv, W
         if c == 0:   # added to what was there, in fp32
             ref_k, ref_v = ref_k + 1.5, ref_v - 2.0
         assert torch.equal(dks[c], ref_k) and torch.equal(dvs[c], ref_v), c
+    # the same launch as the LAST block of the chunks' sums: the totals (chunk 0: what its fp32 buffers held + this
+    # block; the others: this block alone) leave rounded to bf16, in [B,S,H,D] memory here, and the fp32 buffers are
+    # only read -- the same fp32 sums as above, rounded once
+    old_k = [torch.full(t.shape, 1.5, dtype=torch.float32, device=device) if i == 0 else None for i, t in enumerate(ks)]
+    old_v = [torch.full(t.shape, -2.0, dtype=torch.float32, device=device) if i == 0 else None for i, t in enumerate(ks)]
+    fin_k = [torch.empty(B, Sc, Hkv, D, dtype=torch.bfloat16, device=device).transpose(1, 2) for _ in ks]
+    fin_v = [torch.empty(B, Sc, Hkv, D, dtype=torch.bfloat16, device=device).transpose(1, 2) for _ in ks]
+    # (dq is asked for again so that delta comes from the same place, the dQ kernel's prologue, bit for bit)
+    ops.attn_bwd_chunks(dod, qd, ks, vs, lse, scale, causal, q_off, torch.empty_like(qd), old_k, old_v,
+                        dkv_accumulate=[i == 0 for i in range(n)], out=out, dk_finals=fin_k, dv_finals=fin_v)
+    assert torch.equal(old_k[0], torch.full_like(old_k[0], 1.5)) and torch.equal(old_v[0], torch.full_like(old_v[0], -2.0))
+    for c in range(n):
+        assert torch.equal(fin_k[c], dks[c].to(torch.bfloat16)) and torch.equal(fin_v[c], dvs[c].to(torch.bfloat16)), c
     w_dq, contrib = OR.rank_backward(do[:, :, sl].float(), q[:, :, sl].float(), kf, vf, out.float().cpu(), lse.cpu(), r, scale, causal)
     fold = lambda t: t.view(B, Hkv, rep, Sc, D).sum(2)
     assert maxabs(delta, (do[:, :, sl].float() * out.float().cpu()).sum(-1)) <= 5e-2

@@ -98,7 +98,8 @@ def fake_attn_fwd_chunks(q, ks, vs, sm_scale, causal, q_offset=0, out=None, lse=
 
 
 def fake_attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale, causal, q_offset=0, dq=None, dks=None, dvs=None, dq_accumulate=False,
-                         dkv_accumulate=None, out=None, delta=None, rope=None, q_pos_offset=0, k_pos_offset=0):
+                         dkv_accumulate=None, out=None, delta=None, rope=None, q_pos_offset=0, k_pos_offset=0,
+                         dk_finals=None, dv_finals=None):
     assert rope is None
     Sc = ks[0].size(2)
     qf, kf, vf, rep = _expand(q, torch.cat(ks, 2), torch.cat(vs, 2))
@@ -113,9 +114,15 @@ def fake_attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale, causal, q_offset=0, dq=
         b_dq = ds @ kf * sm_scale
         dq.add_(b_dq) if dq_accumulate else dq.copy_(b_dq)
     for c in range(len(ks)):
+        sl = slice(c * Sc, (c + 1) * Sc)
+        if dk_finals is not None and dk_finals[c] is not None:
+            # the block that completes the chunk's sums: total = sums so far (if any) + this block, cast once
+            add = dkv_accumulate is not None and dkv_accumulate[c]
+            dk_finals[c].copy_(b_dk[:, :, sl] + (dks[c] if add else 0))
+            dv_finals[c].copy_(b_dv[:, :, sl] + (dvs[c] if add else 0))
+            continue
         if dks is None or dks[c] is None:
             continue
-        sl = slice(c * Sc, (c + 1) * Sc)
         if dkv_accumulate is not None and dkv_accumulate[c]:
             dks[c].add_(b_dk[:, :, sl])
             dvs[c].add_(b_dv[:, :, sl])
@@ -139,6 +146,7 @@ def ring(monkeypatch, request):
     monkeypatch.setattr(ops, "attn_fwd_chunks", fake_attn_fwd_chunks)
     monkeypatch.setattr(ops, "attn_bwd_chunks", fake_attn_bwd_chunks)
     monkeypatch.setattr(ops, "chunks_fit_one_launch", lambda ks, vs: request.param == "one_launch_per_rank")
+    monkeypatch.setattr(ops, "FINAL_TOTAL_DTYPES", (torch.bfloat16, torch.float32))   # the stand-in handles fp32 as well
     yield pgm, cp
     pgm.setup_process_group_manager(1, 1, 1, 1)
 
@@ -205,6 +213,36 @@ def test_non_causal_ring_forward_and_backward(ring, W):
         (out * do).sum().backward()
         w_o, w_q, w_k, w_v = _want(q, k, v, do, False)
         assert close(out, w_o) and close(qd.grad, w_q) and close(kd.grad, w_k) and close(vd.grad, w_v)
+
+
+def test_last_reader_hands_back_the_totals_itself(ring, monkeypatch):
+    """One launch per rank: the rank whose block completes a chunk's dK / dV (every rank that read the chunk has added
+    its block) writes the rounded totals in the same call, so a whole backward needs no cast pass at all; when the
+    ranks' losses are differentiated one at a time no block is ever the last of its pass, and the chunks' own nodes
+    cast the sums they hold."""
+    pgm, cp = ring
+    from picotron_amd import ops
+    if not ops.chunks_fit_one_launch(None, None):
+        pytest.skip("the per-step ring keeps the reference's shape: fp32 sums, cast at the end")
+    casts = {"n": 0}
+    real = ops.convert_f32
+    monkeypatch.setattr(ops, "convert_f32", lambda *a, **k: (casts.__setitem__("n", casts["n"] + 1), real(*a, **k))[1])
+    W = 4
+    mgr = pgm.setup_process_group_manager(1, W, 1, 1)
+    q, k, v, do = _inputs(W, 21)
+    Sc = q.size(2) // W
+    w_o, w_q, w_k, w_v = _want(q, k, v, do, True)
+    qd, kd, vd = (t.clone().requires_grad_() for t in (q, k, v))
+    out = torch.cat(_play(mgr, cp, qd, kd, vd, True, W), dim=2)
+    (out * do).sum().backward()
+    assert casts["n"] == 0
+    assert close(qd.grad, w_q) and close(kd.grad, w_k) and close(vd.grad, w_v)
+    qd, kd, vd = (t.clone().requires_grad_() for t in (q, k, v))
+    outs = _play(mgr, cp, qd, kd, vd, True, W)
+    for r in (2, 0, 3, 1):
+        (outs[r] * do[:, :, r * Sc:(r + 1) * Sc]).sum().backward()
+    assert casts["n"] > 0
+    assert close(qd.grad, w_q) and close(kd.grad, w_k) and close(vd.grad, w_v)
 
 
 def test_missing_chunk_raises_instead_of_delivering_zeros(ring):
