@@ -449,8 +449,14 @@ def train_step_extra(torch, which="smollm_1p7b", steps=10, warmup=3, adamw="fp32
         opt.step()
         return loss
 
+    # the loss of the very first step (random init, nothing updated yet) is a function of the seed and the kernels
+    # alone: reproducible to ~1e-2 across builds and close to ln(vocab); the loss after a dozen bf16 updates on one
+    # batch is not (it differs by +-1 between builds), so it is not reported
+    first_loss = None
     for _ in range(warmup):
         loss = step()
+        if first_loss is None:
+            first_loss = loss.item()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -460,7 +466,8 @@ def train_step_extra(torch, which="smollm_1p7b", steps=10, warmup=3, adamw="fp32
     n = get_num_params(model)
     tok_s = mbs * seq / dt
     fpt = flops_per_token(n, cfg.num_hidden_layers, cfg.hidden_size, seq)
-    res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_after": round(loss.item(), 4),
+    res = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(dt * 1e3, 2), "params": n, "loss_first_step": round(first_loss, 4),
+           "ln_vocab": round(math.log(cfg.vocab_size), 4),
            "mfu_vs_2.5PF": round(tok_s * fpt / MI355X_BF16_DENSE_FLOPS, 4), "steps": steps,
            "adamw_state": layouts[adamw][1],
            "note": "attention / RMSNorm with the residual adds / RoPE / SwiGLU / cross-entropy / AdamW on the HIP kernels; "
