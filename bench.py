@@ -133,6 +133,24 @@ class RingBench:
         ops.attn_bwd(do, q, k, v, self.lse[r], self.delta[r], self.scale, True, r * self.Sc, self.dq_acc[r], dk, dv,
                      dkv_accumulate=True, out=out)
 
+    def step_one_rank_last_reader(self, r):
+        """Forward + backward of cp rank r alone, with the gradient traffic that rank has in a real ring when it is the
+        last rank to contribute to every chunk it reads (context_parallel.py:74-108 with is_causal: chunk c collects the
+        blocks of ranks c, c+1, ... in that order, so the highest rank comes last): dq leaves in bf16; for the chunks of
+        the ranks below, the fp32 sums that arrived with the chunk are read and the rounded total is written; the rank's
+        own chunk, which nobody else reads, is written in bf16 directly.  One launch per direction over the chunk list."""
+        ops, Sc = self.ops, self.Sc
+        q, k, v, do, out, dk, dv = self._views(r)
+        ks = [self.k[:, :, c * Sc:(c + 1) * Sc] for c in range(r + 1)]
+        vs = [self.v[:, :, c * Sc:(c + 1) * Sc] for c in range(r + 1)]
+        ops.attn_fwd_chunks(q, ks, vs, self.scale, True, r * Sc, out=out, lse=self.lse[r])
+        sums_k = [self.dk_acc[:, :, c * Sc:(c + 1) * Sc] if c < r else None for c in range(r + 1)]
+        sums_v = [self.dv_acc[:, :, c * Sc:(c + 1) * Sc] if c < r else None for c in range(r + 1)]
+        ops.attn_bwd_chunks(do, q, ks, vs, self.lse[r], self.scale, True, r * Sc, self.dq_b[:, :, r * Sc:(r + 1) * Sc],
+                            sums_k, sums_v, dkv_accumulate=[c < r for c in range(r + 1)], out=out, delta=self.delta[r],
+                            dk_finals=[self.dk_b[:, :, c * Sc:(c + 1) * Sc] for c in range(r + 1)],
+                            dv_finals=[self.dv_b[:, :, c * Sc:(c + 1) * Sc] for c in range(r + 1)])
+
     def step_ranks_parallel(self):
         """One launch per rank and direction, like step(), but the ranks' launches are independent branches: rank r's
         forward, delta pre-pass and dQ kernel run on stream r, the dK/dV launches (which add into shared chunks) follow
@@ -764,7 +782,14 @@ def main():
         extras["rank3_of_4_alone"] = {"TFLOP/s": round(r3_flops / (ms_r3 * 1e-3) / 1e12, 2), "us_per_step": round(ms_r3 * 1e3, 2),
                                       "flops": r3_flops,
                                       "frac_of_mfma_peak": round(r3_flops / (ms_r3 * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
-                                      "schedule": "the last rank's share alone: 256 queries of every head over chunks 0..3"}
+                                      "schedule": "the last rank's share alone: 256 queries of every head over chunks 0..3; fp32 dq, "
+                                                  "fp32 dk / dv sums of all four chunks read, added to and written back"}
+        ms_r3l, _ = graph_time(torch, lambda: rb.step_one_rank_last_reader(3), max(args.steps // 10, 10), per_graph=10)
+        extras["rank3_of_4_alone_as_last_reader"] = {
+            "TFLOP/s": round(r3_flops / (ms_r3l * 1e-3) / 1e12, 2), "us_per_step": round(ms_r3l * 1e3, 2),
+            "frac_of_mfma_peak": round(r3_flops / (ms_r3l * 1e-3) / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "schedule": "the same share with the gradient traffic rank 3 has in the ring, where it contributes last to every chunk: "
+                        "bf16 dq; fp32 sums of chunks 0..2 read and their rounded totals written; its own chunk written in bf16"}
         extras["ring_attention_api"] = ring_api_extra(torch, ops, rb)
         ms_ring, _ = graph_time(torch, rb.step_per_ring_step, max(args.steps // 4, 10))
         extras["one_launch_per_ring_step"] = {"TFLOP/s": round(total_flops / (ms_ring * 1e-3) / 1e12, 2), "ms_per_step": round(ms_ring, 4),
