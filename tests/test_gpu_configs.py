@@ -218,6 +218,28 @@ def test_configs4_long_context_rank7_of_8(ops, device):
     assert maxabs(out1[:, qs], r_o) <= 2e-2 and maxabs(lse1[:, qs], r_l) <= 1e-3
     assert rel_l2(dq1[:, qs], r_dq) <= 1e-2 and rel_l2(dk1[:, 1:2], r_dk) <= 1e-2 and rel_l2(dv1[:, 1:2], r_dv) <= 1e-2
 
+    # the same step as ONE launch per direction over the eight chunks as separate tensors, RoPE inside the kernels:
+    # q rotated in the forward's prologue at the rank's positions, dq / dk un-rotated in the backward's epilogues at
+    # every chunk's own positions.  Forward: bit-equal to the one-tensor launch on the rotated q it leaves behind.
+    ks = [k_rot[:, :, c * Sc:(c + 1) * Sc].contiguous() for c in range(W)]
+    vs = [v[:, :, c * Sc:(c + 1) * Sc].contiguous() for c in range(W)]
+    out3, lse3, q_rot3 = ops.attn_fwd_chunks(q, ks, vs, scale, True, r * Sc, rope=(cos_d, sin_d), q_pos_offset=r * Sc,
+                                              want_q_rot=True)
+    assert maxabs(q_rot3, q_rot) <= 2 ** -5      # one bf16 ulp of a rotated element (fp32 rotation, one rounding)
+    o_chk, l_chk = ops.attn_fwd(q_rot3, k_rot, v, scale, True, r * Sc)
+    assert torch.equal(out3, o_chk) and torch.equal(lse3, l_chk)
+    assert maxabs(out3, out1) <= 2e-2 and maxabs(lse3, lse1) <= 2e-3
+    dq3 = torch.empty_like(dq1)
+    dks3 = [torch.empty(1, Hkv, Sc, D, dtype=torch.float32, device=device) for _ in range(W)]
+    dvs3 = [torch.empty_like(t) for t in dks3]
+    ops.attn_bwd_chunks(do, q_rot3, ks, vs, lse3, scale, True, r * Sc, dq3, dks3, dvs3, out=out3,
+                        rope=(cos_d, sin_d), q_pos_offset=r * Sc, k_pos_offset=0)
+    # reference for the un-rotated gradients: rotate the one-tensor launch's gradients back with the RoPE kernel
+    dq_want = ops.rope(dq1, cos_d, sin_d, pos_offset=r * Sc, inverse=True)
+    dk_want = ops.rope(dk1, cos_d, sin_d, inverse=True)
+    assert rel_l2(dq3, dq_want) <= 1e-2
+    assert rel_l2(torch.cat(dks3, 2), dk_want) <= 1e-2 and rel_l2(torch.cat(dvs3, 2), dv1) <= 1e-2
+
 
 def test_elementwise_properties_at_full_sizes(ops, device):
     """Size-independent properties at the SmolLM-1.7B / Llama-2-7B step's sizes: RoPE is an isometry and its backward
