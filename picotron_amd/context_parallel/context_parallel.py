@@ -176,7 +176,7 @@ class RingAttentionFunc(torch.autograd.Function):
         if not _per_step() and contiguous_positions and ops.chunks_fit_one_launch(ks, vs):
             q_off = (rank - order[0]) * Sq if is_causal else 0
             out, lse, q_rot = ops.attn_fwd_chunks(q, ks, vs, sm_scale, is_causal, q_off, out_dtype=q.dtype, bshd_out=True,
-                                                  rope=cs, q_pos_offset=q_pos, want_q_rot=rope is not None)
+                                                  rope=cs, q_pos_offset=q_pos, want_q_rot=rope is not None, checked=True)
             ctx.one_launch = (order, q_off)
             ctx.save_for_backward(q_rot if rope is not None else q, out, lse)
             return out
@@ -277,7 +277,8 @@ class RingAttentionFunc(torch.autograd.Function):
                                 [g[1] for g in got], dkv_accumulate=[g[2] for g in got], out=out, rope=cs,
                                 q_pos_offset=q_pos, k_pos_offset=q_pos - q_off if is_causal else 0,
                                 dk_finals=[fin[c][0] if fin[c] is not None else None for c in order],
-                                dv_finals=[fin[c][1] if fin[c] is not None else None for c in order])
+                                dv_finals=[fin[c][1] if fin[c] is not None else None for c in order],
+                                checked=True)   # (the forward asked chunks_fit_one_launch about these same tensors)
             return (dq,) + nothing[1:]
 
         delta = ops.attn_bwd_preprocess(dout, out)

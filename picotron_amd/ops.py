@@ -318,11 +318,13 @@ def chunks_fit_one_launch(ks, vs) -> bool:
     k0, v0 = ks[0], vs[0]
     if k0.dim() != 4 or (len(ks) > 1 and k0.size(2) % 128 != 0):
         return False
-    for k, v in zip(ks, vs):
-        if (k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16 or k.shape != k0.shape or v.shape != k0.shape
-                or k.stride() != k0.stride() or v.stride() != v0.stride() or k.stride(-1) != 1 or v.stride(-1) != 1
-                or any(s % 8 for s in k.stride()[:3]) or any(s % 8 for s in v.stride()[:3])
-                or k.data_ptr() % 16 or v.data_ptr() % 16 or not k.is_cuda or not v.is_cuda):
+    shape, ksd, vsd, bf16 = k0.shape, k0.stride(), v0.stride(), torch.bfloat16
+    if (v0.dim() != 4 or ksd[3] != 1 or vsd[3] != 1 or ksd[0] % 8 or ksd[1] % 8 or ksd[2] % 8
+            or vsd[0] % 8 or vsd[1] % 8 or vsd[2] % 8):
+        return False
+    for k, v in zip(ks, vs):      # (this runs once per attention call of every layer: kept flat)
+        if (k.dtype != bf16 or v.dtype != bf16 or k.shape != shape or v.shape != shape or k.stride() != ksd
+                or v.stride() != vsd or k.data_ptr() % 16 or v.data_ptr() % 16 or not k.is_cuda or not v.is_cuda):
             return False
     return True
 
@@ -352,12 +354,12 @@ def _chunk_desc(q, ks, vs, o, sm_scale, causal, q_offset) -> AttnDesc:
 
 def attn_fwd_chunks(q, ks, vs, sm_scale: float, causal: bool, q_offset: int = 0, out=None, lse=None, merge: bool = False,
                     out_dtype=torch.bfloat16, bshd_out: bool = False, rope=None, q_pos_offset: int = 0,
-                    want_q_rot: bool = False):
+                    want_q_rot: bool = False, checked: bool = False):
     """attn_fwd over K / V given as lists of chunk tensors (see chunks_fit_one_launch) that follow each other along the
     key axis: key j sits at position j of the concatenation, which is never materialised.  rope = (cos, sin): q is
     rotated inside the kernel (the chunks' k must be rotated already).  Returns (out, lse, q_rot or None)."""
     _dev(q, out, lse)
-    if not chunks_fit_one_launch(ks, vs):
+    if not checked and not chunks_fit_one_launch(ks, vs):     # checked: the caller has asked chunks_fit_one_launch already
         raise RuntimeError("attn_fwd_chunks: the chunks do not fit one launch (see chunks_fit_one_launch)")
     q = _attn_in(q, "q")
     B, Hq, Sq, D = q.shape
@@ -386,7 +388,7 @@ def attn_fwd_chunks(q, ks, vs, sm_scale: float, causal: bool, q_offset: int = 0,
 
 def attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale: float, causal: bool, q_offset: int = 0, dq=None, dks=None, dvs=None,
                     dq_accumulate: bool = False, dkv_accumulate=None, out=None, delta=None, rope=None,
-                    q_pos_offset: int = 0, k_pos_offset: int = 0, dk_finals=None, dv_finals=None):
+                    q_pos_offset: int = 0, k_pos_offset: int = 0, dk_finals=None, dv_finals=None, checked: bool = False):
     """attn_bwd over a chunk list.  dks / dvs: per chunk a gradient buffer (all of one dtype and stride triple) or None
     (not wanted); dkv_accumulate: per chunk, add to the fp32 buffer instead of writing it.  dq None: not wanted.  With
     `out` (forward output) delta is computed inside the call, otherwise `delta` must be given.  rope = (cos, sin): q and
@@ -395,7 +397,7 @@ def attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale: float, causal: bool, q_offse
     total -- the fp32 sums in dks / dvs (if the chunk's dkv_accumulate flag is set) plus this block -- is written there,
     rounded once; the fp32 buffers are only read.  Returns delta."""
     _dev(dout, q, lse, dq, out, delta)
-    if not chunks_fit_one_launch(ks, vs):
+    if not checked and not chunks_fit_one_launch(ks, vs):
         raise RuntimeError("attn_bwd_chunks: the chunks do not fit one launch (see chunks_fit_one_launch)")
     q, dout = _attn_in(q, "q"), _attn_in(dout, "dout")
     B, Hq, Sq, D = q.shape

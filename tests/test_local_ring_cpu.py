@@ -89,7 +89,7 @@ def _full_scores(q, k_all, sm_scale, causal, q_offset):
 
 
 def fake_attn_fwd_chunks(q, ks, vs, sm_scale, causal, q_offset=0, out=None, lse=None, merge=False, out_dtype=torch.bfloat16,
-                         bshd_out=False, rope=None, q_pos_offset=0, want_q_rot=False):
+                         bshd_out=False, rope=None, q_pos_offset=0, want_q_rot=False, checked=False):
     """All listed chunks in one go: softmax over their concatenation, query i at position q_offset + i."""
     assert rope is None and not merge
     qf, kf, vf, _ = _expand(q, torch.cat(ks, 2), torch.cat(vs, 2))
@@ -99,7 +99,7 @@ def fake_attn_fwd_chunks(q, ks, vs, sm_scale, causal, q_offset=0, out=None, lse=
 
 def fake_attn_bwd_chunks(dout, q, ks, vs, lse, sm_scale, causal, q_offset=0, dq=None, dks=None, dvs=None, dq_accumulate=False,
                          dkv_accumulate=None, out=None, delta=None, rope=None, q_pos_offset=0, k_pos_offset=0,
-                         dk_finals=None, dv_finals=None):
+                         dk_finals=None, dv_finals=None, checked=False):
     assert rope is None
     Sc = ks[0].size(2)
     qf, kf, vf, rep = _expand(q, torch.cat(ks, 2), torch.cat(vs, 2))
