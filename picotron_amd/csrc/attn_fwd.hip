@@ -400,7 +400,10 @@ int launch(const FwdParams& p, hipStream_t s) {
     return fail(PICO_ERR_LAUNCH, "pico_attn_fwd: cannot reserve %zu bytes of LDS", C::kLdsBytes);
   const int n_qtiles = (p.a.Sq + C::BM - 1) / C::BM;
   FwdParams q = p;
-  q.pair_order = p.a.causal && n_qtiles >= 2 && static_cast<int64_t>(p.a.Hq) * p.a.B * n_qtiles <= 512;
+  // (the pairing needs two workgroups per CU: at head_dim 128 the eight-wave kernel has one, the launch is two
+  // generations of workgroups and longest-first is the better order -- 160 -> 137 us at B1 H32 S4096)
+  constexpr bool kTwoPerCu = !(D >= 128 && NW == 8);
+  q.pair_order = kTwoPerCu && p.a.causal && n_qtiles >= 2 && static_cast<int64_t>(p.a.Hq) * p.a.B * n_qtiles <= 512;
   hipLaunchKernelGGL((attn_fwd_kernel<D, QB, NW, KT, KS>), dim3(p.a.Hq * p.a.B, n_qtiles), dim3(C::kThreads), C::kLdsBytes, s, q);
   return PICO_OK;
 }
@@ -562,7 +565,8 @@ int run_fwd(const char* fn, const pico_attn_desc* desc, const void* q, const pic
     else rc = launch<64, 1, 4, 128, 2>(p, s);
   } else {
     const int64_t heads = static_cast<int64_t>(desc->B) * desc->Hq;
-    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<128, 1, 8, 128>(p, s);
+    // (64-key staged tiles: 0.5-4 % faster than 128-key ones at every size measured)
+    if (heads * ((desc->Sq + 255) / 256) >= 256) rc = launch<128, 1, 8, 64>(p, s);
     else rc = launch<128, 1, 4, 64>(p, s);
   }
   if (rc) return rc;
