@@ -1051,7 +1051,12 @@ int run_bwd(const char* fn, const pico_attn_desc* desc, const void* q, const pic
       // the forward's rules: eight waves per workgroup also for rectangular launches (every query sees at least as many
       // keys as there are queries) with fewer workgroups than the square ones need
       const bool rectangular = !desc->causal || desc->q_offset >= desc->Sq;
-      if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
+      // several generations of workgroups over short key ranges (a few trips each): two four-wave workgroups per CU hide
+      // each other's prologues and epilogues, which one eight-wave workgroup per CU cannot (B8 S768 51.3 -> 44.3 us,
+      // B16 S512 54.4 -> 48.1, B8 S1024 78.5 -> 72.9, B8 S1536 147.8 -> 144.3; from S2048 on, and with 512 workgroups,
+      // the eight-wave kernel is level or ahead)
+      if (groups(256) >= 768 && visible_keys <= 1536) rc = launch_dq<64, 4, 64>(p, s);
+      else if (groups(256) >= 512) rc = launch_dq<64, 8, 64>(p, s);
       else if (groups(128) >= 512) {
         if (rectangular && groups(256) >= 256) rc = launch_dq<64, 8, 64>(p, s);
         else rc = launch_dq<64, 4, 64>(p, s);

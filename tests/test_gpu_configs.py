@@ -136,6 +136,7 @@ def test_head_dim_128_large_launch_ragged_lengths(ops, device, Sq, Sk, q_offset,
     (4, 32, 256, 256, 0, True),        # rank 0 of 4: key split, four waves (few keys, not rectangular)
     (1, 8, 1024, 700, 0, False),       # dense: key split, eight waves
     (8, 32, 256, 1024, 768, True),     # rectangular with 256 workgroups of 256 queries: the 8-wave kernels
+    (8, 32, 700, 700, 0, True),        # several generations of short tiles: 8-wave forward, 4-wave dQ
 ])
 def test_head_dim_64_every_launch_size_class(ops, device, B, Hkv, Sq, Sk, q_offset, causal):
     """head_dim 64 at 32 query heads: the library picks 8-wave, 4-wave or key-split workgroups (of eight or four waves) by
