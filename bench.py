@@ -54,7 +54,7 @@ def parse():
     ap.add_argument("--no-train", action="store_true", help="skip the SmolLM-1.7B- and Llama-2-7B-shaped training steps")
     ap.add_argument("--train-step", choices=["smollm_1p7b", "llama2_7b"], default=None,
                     help="run only that training step (for a kernel trace of it) and print its figures")
-    ap.add_argument("--probe", nargs="?", const="configs1", default=None, choices=["configs1", "configs4"],
+    ap.add_argument("--probe", nargs="?", const="configs1", default=None, choices=["configs1", "configs4", "ring_api"],
                     help="counter probe: a few launches of a plain copy of known size and of each attention kernel "
                          "at the bench shape (configs1) or at configs[4]'s shape (rank 7 of 8, head_dim 128), nothing else "
                          "(for rocprofv3 --pmc)")
@@ -232,7 +232,7 @@ class RingBench:
         self.dv = ops.convert_f32(self.dv_acc, torch.bfloat16)
 
 
-def ring_api_extra(torch, ops, rb, iters=20):
+def ring_api_extra(torch, ops, rb, iters=20, eager_only=False):
     """The public API at configs[1]: ring_attention() (RingAttentionFunc, context_parallel.py:14-51) forward and
     backward for the four virtual cp ranks -- every rank's own q / k / v chunk tensors (leaves that require gradients),
     the ranks played in ascending order, one backward over all of them.  Autograd, the mailbox, the chunks' publishing
@@ -244,7 +244,9 @@ def ring_api_extra(torch, ops, rb, iters=20):
     W, Sc = rb.W, rb.Sc
     mgr = pgm.setup_process_group_manager(1, W, 1, 1)
     leaves = [[t[:, :, r * Sc:(r + 1) * Sc].clone().requires_grad_() for t in (rb.q, rb.k, rb.v)] for r in range(W)]
-    dos = [rb.do[:, :, r * Sc:(r + 1) * Sc].clone() for r in range(W)]
+    # the output gradient in the memory layout of the output ([B,S,H,D], as it arrives from the o_proj's backward through
+    # the free transpose + reshape of model.py:160): a gradient laid out otherwise makes the backward copy `out` first
+    dos = [rb.do[:, :, r * Sc:(r + 1) * Sc].transpose(1, 2).contiguous().transpose(1, 2) for r in range(W)]
     total_flops = sum(rb.flops())
 
     def step():
@@ -265,6 +267,8 @@ def ring_api_extra(torch, ops, rb, iters=20):
     res = {"what": "ring_attention() forward + backward over the 4 virtual ranks of configs[1] through autograd "
                    "(one launch per rank and direction over the chunk list; PICO_RING_PER_STEP=1 gives the per-step shape)"}
     try:
+        if eager_only:
+            raise RuntimeError("not asked for")
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
@@ -694,6 +698,12 @@ def main():
                                    "(rank 7 of 8: 4096 queries x 32768 keys, GQA 32/8, head_dim 128)"}))
         return
     rb = RingBench(torch, ops)
+    if args.probe == "ring_api":
+        # the public API's step (ring_attention() forward + backward over the four virtual ranks), launched eagerly a few
+        # times so that a kernel trace shows what one step consists of
+        res = ring_api_extra(torch, ops, rb, iters=20, eager_only=True)
+        print(json.dumps({"probe": "ring_attention() through autograd over the 4 virtual ranks of configs[1], eager", **res["eager"]}))
+        return
     if args.probe:
         # plain copy of 64 MiB fp32 (read 64 MiB, write 64 MiB) as the scale for the HBM counters
         src = torch.randn(16, 1024, 1024, dtype=torch.float32, device="cuda").view(1, 16, 1024, 1024)
